@@ -58,7 +58,7 @@ FLAGS = [
 ]
 PLAIN_SOURCES = {"core": "core.hip", "gemm": "gemm.hip", "gemm_tile": "gemm_tile.hip", "sampling": "sampling.hip",
                  "rowwise": "rowwise.hip", "sink_attention": "sink_attention.hip",
-                 "linear_recurrence": "linear_recurrence.hip", "rows_attention": "rows_attention.hip"}
+                 "linear_recurrence": "linear_recurrence.hip", "rows_attention": "rows_attention.hip", "moe": "moe.hip"}
 ATTENTION_SOURCE = "attention.hip"
 # head sizes compiled by build_all: the tests' models, the kernel tests and the benchmark's
 DEFAULT_HEAD_DIMS = (16, 32, 48, 64, 96, 128, 160, 224, 256)

@@ -4,7 +4,9 @@
 // the logit cap, the mean of two RMS-normed rows, the RMS norm of whole query / key
 // projections fused with the cache write, residual add + Dynamic Tanh, the erf GELU, a sigmoid
 // gate, biased projections into cache rows, the low-rank query step with the latent cache row,
-// and the rotation of one part of every head.
+// the rotation of one part of every head, the RMS norm of a branch's output as it joins the
+// stream, the RMS norm of the stream with a weight kept as a distance from a constant, the RMS
+// norm of every query / key vector with rotation and cache write, squared ReLU, and a scale.
 // Statistics, gates and the residual stream are float32; T is the activation type.
 #include "common.h"
 
@@ -653,5 +655,219 @@ CW_EXPORT int cw_rotate_part(const void* src, int dtype, int64_t src_stride, int
     hipLaunchKernelGGL(rotate_part_kernel<bf16_t>, grid, block, 0, stream, (const bf16_t*)src, src_stride, src_head, src_off,
                        (bf16_t*)dst, dst_stride, dst_head, dst_off, heads, n, rdims, positions, freq);
   else return CW_ERR_DTYPE;
+  return cw_launch_status();
+}
+
+// ---------------------------------------------------------------- a branch's output, normed, joins the stream
+// For a block that norms what a sublayer gives back and not what it reads:
+//   resid[t, :] += scale * branch[t, :] / sqrt(mean(branch[t, :]^2) + eps) * (w_offset + w)
+// and image[t, :] = resid[t, :] in the activation type (what the next sublayer reads); image may be
+// nullptr, and so may branch (then nothing is added and the image alone is made). float32 inside.
+template <typename T, typename WT>
+__global__ __launch_bounds__(256) void branch_norm_add_kernel(float* __restrict__ resid, const T* __restrict__ branch,
+                                                              const WT* __restrict__ w, float w_offset, float eps, float scale,
+                                                              T* __restrict__ image, int H) {
+  __shared__ float scratch[4];
+  const int64_t t = blockIdx.x;
+  float* x = resid + t * H;
+  const T* b = branch ? branch + t * H : nullptr;
+  T* im = image ? image + t * H : nullptr;
+  float inv = 0.0f;
+  if (b) {
+    float ss = 0.0f;
+    for (int j = threadIdx.x; j < H; j += 256) { const float v = cw_to_float(b[j]); ss += v * v; }
+    inv = scale / sqrtf(block_sum_256(ss, scratch) / (float)H + eps);
+  }
+  for (int j = threadIdx.x; j < H; j += 256) {
+    float v = x[j];
+    if (b) {
+      v += cw_to_float(b[j]) * inv * (w_offset + cw_to_float(w[j]));
+      x[j] = v;
+    }
+    if (im) im[j] = cw_from_float<T>(v);
+  }
+}
+
+CW_EXPORT int cw_branch_norm_add(float* resid, const void* branch, const void* w, int w_dtype, float w_offset, float eps,
+                                 float scale, void* image, int dtype, int T, int H, hipStream_t stream) {
+  if (T < 0 || H <= 0 || !resid || (branch && !w)) return CW_ERR_ARG;
+  if (T == 0 || (!branch && !image)) return CW_OK;
+  dim3 grid(T), block(256);
+#define CW_LAUNCH(T_, WT_)                                                                                           \
+  hipLaunchKernelGGL((branch_norm_add_kernel<T_, WT_>), grid, block, 0, stream, resid, (const T_*)branch, (const WT_*)w, \
+                     w_offset, eps, scale, (T_*)image, H)
+  const int wt = branch ? w_dtype : dtype;
+  if (dtype == CW_F32 && wt == CW_F32) CW_LAUNCH(float, float);
+  else if (dtype == CW_BF16 && wt == CW_BF16) CW_LAUNCH(bf16_t, bf16_t);
+  else if (dtype == CW_BF16 && wt == CW_F32) CW_LAUNCH(bf16_t, float);
+  else return CW_ERR_DTYPE;
+#undef CW_LAUNCH
+  return cw_launch_status();
+}
+
+// ---------------------------------------------------------------- RMS norm of the stream, weight as an offset
+// out[i, :] = resid[r, :] / sqrt(mean(resid[r, :]^2) + eps) * (w_offset + w), r = rows ? rows[i] : i;
+// the product is made in float32 and rounded once. The stream is left as it is.
+template <typename T, typename WT>
+__global__ __launch_bounds__(256) void stream_norm_kernel(const float* __restrict__ resid, const WT* __restrict__ w,
+                                                          float w_offset, float eps, T* __restrict__ out,
+                                                          const int* __restrict__ rows, int H) {
+  __shared__ float scratch[4];
+  const int64_t i = blockIdx.x;
+  const float* x = resid + (int64_t)(rows ? rows[i] : (int)i) * H;
+  float ss = 0.0f;
+  for (int j = threadIdx.x; j < H; j += 256) ss += x[j] * x[j];
+  const float inv = 1.0f / sqrtf(block_sum_256(ss, scratch) / (float)H + eps);
+  for (int j = threadIdx.x; j < H; j += 256) out[i * H + j] = cw_from_float<T>(x[j] * inv * (w_offset + cw_to_float(w[j])));
+}
+
+CW_EXPORT int cw_stream_norm(const float* resid, const void* w, int w_dtype, float w_offset, float eps, void* out, int dtype,
+                             const int* rows, int n, int H, hipStream_t stream) {
+  if (n < 0 || H <= 0 || !resid || !w || !out) return CW_ERR_ARG;
+  if (n == 0) return CW_OK;
+  dim3 grid(n), block(256);
+#define CW_LAUNCH(T_, WT_)                                                                                          \
+  hipLaunchKernelGGL((stream_norm_kernel<T_, WT_>), grid, block, 0, stream, resid, (const WT_*)w, w_offset, eps, (T_*)out, \
+                     rows, H)
+  if (dtype == CW_F32 && w_dtype == CW_F32) CW_LAUNCH(float, float);
+  else if (dtype == CW_BF16 && w_dtype == CW_BF16) CW_LAUNCH(bf16_t, bf16_t);
+  else if (dtype == CW_BF16 && w_dtype == CW_F32) CW_LAUNCH(bf16_t, float);
+  else return CW_ERR_DTYPE;
+#undef CW_LAUNCH
+  return cw_launch_status();
+}
+
+// ---------------------------------------------------------------- per-vector q/k norm, rotation, cache write
+// A row of proj holds a token's query projection (nqv vectors of dim elements from column q_off),
+// its key projection (nkv vectors of dim from k_off) and, unless the values are the keys, its value
+// projection (nv elements from v_off). bias (one element per column of proj, or nullptr) is added
+// first. Every query and key vector by itself is then divided by its root mean square (eps inside
+// the root) and multiplied by qw / kw (dim elements, shared by all vectors; nullptr: no norm), and
+// its first rdims elements are rotated by the token's position: pairs (i, i + rdims / 2), angle =
+// float(position) * freq[i]. Queries are rewritten in place, keys go to k_plane[slot, nkv * dim].
+// Values go to v_plane[slot, nv]: the biased value projection, or with v_from_keys the biased key
+// projection as it was before norm and rotation (nv == nkv * dim). A negative slot writes no
+// cache row. One workgroup a token, one wave a vector at a time; float32 inside.
+#define HN_MAX_DIM 1024
+template <typename T, typename WT, typename BT>
+__global__ __launch_bounds__(256) void headnorm_rope_store_kernel(
+    T* __restrict__ proj, int64_t stride, int q_off, int k_off, int v_off, int nqv, int nkv, int dim, int nv,
+    const BT* __restrict__ bias, const WT* __restrict__ qw, const WT* __restrict__ kw, float eps,
+    const int* __restrict__ positions, const float* __restrict__ freq, int rdims, const int* __restrict__ slots,
+    T* __restrict__ k_plane, T* __restrict__ v_plane, int v_from_keys, int64_t cache_rows) {
+  extern __shared__ float hn_vals[];  // [4 waves][dim]
+  const int64_t t = blockIdx.x;
+  T* row = proj + t * stride;
+  int64_t slot = slots ? (int64_t)slots[t] : -1;
+  if (slot >= cache_rows) slot = -1;
+  const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
+  if (slot >= 0 && v_plane) {
+    const int src = v_from_keys ? k_off : v_off;
+    T* vd = v_plane + slot * nv;
+    for (int j = threadIdx.x; j < nv; j += 256)
+      vd[j] = cw_from_float<T>(cw_to_float(row[src + j]) + (bias ? cw_to_float(bias[src + j]) : 0.0f));
+  }
+  const float pos = positions ? (float)positions[t] : 0.0f;
+  const int half = rdims / 2;
+  float* vals = hn_vals + wave * dim;
+  for (int vec = wave; vec < nqv + nkv; vec += 4) {
+    const bool is_q = vec < nqv;
+    if (!is_q && slot < 0) continue;
+    const int base = is_q ? q_off + vec * dim : k_off + (vec - nqv) * dim;
+    const WT* w = is_q ? qw : kw;
+    float ss = 0.0f;
+    for (int j = lane; j < dim; j += 64) {
+      const float v = cw_to_float(row[base + j]) + (bias ? cw_to_float(bias[base + j]) : 0.0f);
+      vals[j] = v;
+      ss += v * v;
+    }
+    const float inv = w ? 1.0f / sqrtf(cw_wave_sum(ss) / (float)dim + eps) : 1.0f;
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront", "local");
+    __builtin_amdgcn_wave_barrier();
+    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront", "local");
+    T* dst = is_q ? row + base : k_plane + slot * ((int64_t)nkv * dim) + (int64_t)(vec - nqv) * dim;
+    for (int j = lane; j < dim; j += 64) {
+      float v;
+      if (j < rdims) {
+        const int i = j < half ? j : j - half;
+        const float a = vals[i] * inv * (w ? cw_to_float(w[i]) : 1.0f);
+        const float b = vals[i + half] * inv * (w ? cw_to_float(w[i + half]) : 1.0f);
+        float s, c;
+        sincosf(pos * freq[i], &s, &c);
+        v = j < half ? a * c - b * s : b * c + a * s;
+      } else {
+        v = vals[j] * inv * (w ? cw_to_float(w[j]) : 1.0f);
+      }
+      dst[j] = cw_from_float<T>(v);
+    }
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront", "local");
+    __builtin_amdgcn_wave_barrier();
+    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront", "local");
+  }
+}
+
+CW_EXPORT int cw_headnorm_rope_store(void* proj, int dtype, int64_t stride, int q_off, int k_off, int v_off, int nqv, int nkv,
+                                     int dim, int nv, const void* bias, int b_dtype, const void* qw, const void* kw,
+                                     int w_dtype, float eps, const int* positions, const float* freq, int rdims,
+                                     const int* slots, void* k_plane, void* v_plane, int v_from_keys, int64_t cache_rows,
+                                     int T, hipStream_t stream) {
+  if (T < 0 || nqv < 0 || nkv < 0 || dim <= 0 || nv < 0 || rdims < 0 || rdims > dim || (rdims & 1)) return CW_ERR_ARG;
+  if (dim > HN_MAX_DIM) return CW_ERR_SIZE;
+  if (q_off < 0 || k_off < 0 || v_off < 0 || q_off + (int64_t)nqv * dim > stride || k_off + (int64_t)nkv * dim > stride)
+    return CW_ERR_ARG;
+  if (v_from_keys ? nv != nkv * dim : v_off + (int64_t)nv > stride) return CW_ERR_ARG;
+  if (!proj || (rdims && (!freq || !positions)) || (slots && nkv && !k_plane) || (slots && nv && !v_plane)) return CW_ERR_ARG;
+  if ((qw == nullptr) != (kw == nullptr)) return CW_ERR_ARG;
+  if (T == 0) return CW_OK;
+  dim3 grid(T), block(256);
+  const size_t lds = (size_t)4 * dim * sizeof(float);
+#define CW_LAUNCH(T_, WT_, BT_)                                                                                          \
+  hipLaunchKernelGGL((headnorm_rope_store_kernel<T_, WT_, BT_>), grid, block, lds, stream, (T_*)proj, stride, q_off, k_off, \
+                     v_off, nqv, nkv, dim, nv, (const BT_*)bias, (const WT_*)qw, (const WT_*)kw, eps, positions, freq, rdims, \
+                     slots, (T_*)k_plane, (T_*)v_plane, v_from_keys, cache_rows)
+  const int wt = qw ? w_dtype : dtype, bt = bias ? b_dtype : dtype;
+  if (dtype == CW_F32 && wt == CW_F32 && bt == CW_F32) CW_LAUNCH(float, float, float);
+  else if (dtype == CW_BF16 && wt == CW_BF16 && bt == CW_BF16) CW_LAUNCH(bf16_t, bf16_t, bf16_t);
+  else if (dtype == CW_BF16 && wt == CW_F32 && bt == CW_BF16) CW_LAUNCH(bf16_t, float, bf16_t);
+  else if (dtype == CW_BF16 && wt == CW_BF16 && bt == CW_F32) CW_LAUNCH(bf16_t, bf16_t, float);
+  else if (dtype == CW_BF16 && wt == CW_F32 && bt == CW_F32) CW_LAUNCH(bf16_t, float, float);
+  else return CW_ERR_DTYPE;
+#undef CW_LAUNCH
+  return cw_launch_status();
+}
+
+// ---------------------------------------------------------------- squared ReLU, in place; a scale, in place
+// x <- max(x, 0)^2, float32 inside.
+template <typename T>
+__global__ void relu_squared_kernel(T* __restrict__ x, int64_t n) {
+  for (int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; i < n; i += (int64_t)gridDim.x * blockDim.x) {
+    const float z = fmaxf(cw_to_float(x[i]), 0.0f);
+    x[i] = cw_from_float<T>(z * z);
+  }
+}
+
+CW_EXPORT int cw_relu_squared(void* x, int dtype, int64_t n, hipStream_t stream) {
+  if (n < 0) return CW_ERR_ARG;
+  if (n == 0) return CW_OK;
+  int64_t blocks = (n + 255) / 256;
+  if (blocks > 262144) blocks = 262144;
+  dim3 grid((unsigned)blocks), block(256);
+  if (dtype == CW_F32) hipLaunchKernelGGL(relu_squared_kernel<float>, grid, block, 0, stream, (float*)x, n);
+  else if (dtype == CW_BF16) hipLaunchKernelGGL(relu_squared_kernel<bf16_t>, grid, block, 0, stream, (bf16_t*)x, n);
+  else return CW_ERR_DTYPE;
+  return cw_launch_status();
+}
+
+// x <- x * s, float32 (logits).
+__global__ void scale_kernel(float* __restrict__ x, int64_t n, float s) {
+  for (int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; i < n; i += (int64_t)gridDim.x * blockDim.x) x[i] *= s;
+}
+
+CW_EXPORT int cw_scale(float* x, int64_t n, float s, hipStream_t stream) {
+  if (n < 0) return CW_ERR_ARG;
+  if (n == 0) return CW_OK;
+  int64_t blocks = (n + 255) / 256;
+  if (blocks > 262144) blocks = 262144;
+  hipLaunchKernelGGL(scale_kernel, dim3((unsigned)blocks), dim3(256), 0, stream, x, n, s);
   return cw_launch_status();
 }

@@ -132,6 +132,19 @@ def _declare(name: str, lib: ctypes.CDLL) -> None:
             "cw_bias_store": [P, I, L, I, I, I, I, I, I, P, I, P, P, P, L, I, P],
             "cw_latent_store": [P, I, L, I, I, I, I, I, I, P, P, I, F, P, P, P, P, P, L, I, P],
             "cw_rotate_part": [P, I, L, L, I, P, L, L, I, I, I, I, P, P, I, P],
+            "cw_branch_norm_add": [P, P, P, I, F, F, F, P, I, I, I, P],
+            "cw_stream_norm": [P, P, I, F, F, P, I, P, I, I, P],
+            "cw_headnorm_rope_store": [P, I, L, I, I, I, I, I, I, I, P, I, P, P, I, F, P, P, I, P, P, P, I, L, I, P],
+            "cw_relu_squared": [P, I, L, P],
+            "cw_scale": [P, L, F, P],
+        },
+        "moe": {
+            "cw_moe_tile_rows": [],
+            "cw_moe_max_tiles": [I, I],
+            "cw_moe_route": [P, P, I, I, I, I, I, I, I, P, P, P],
+            "cw_moe_plan": [P, I, I, P, I, P, I, P, P],
+            "cw_moe_expert_product": [I, P, P, P, I, P, P, P, I, P, I, I, I, I, P],
+            "cw_moe_combine": [P, P, I, I, I, I, P],
         },
         "rows_attention": {
             "cw_rows_attention_key_chunk": [I, I, I, I],
@@ -1820,3 +1833,194 @@ def rows_attention(q, q_strides, out, out_strides, k_plane, v_plane, block_table
         v_row, rows, _ptr(block_tables), block_tables.shape[1], _ptr(ctx_lens), _ptr(cu_q), _ptr(items), n_items, _ptr(sink),
         _ptr(lam), heads, kv_heads, dim, vdim, maps, block_size, MASK_KINDS[mask], int(mask_size), float(scale),
         0 if head_norm_eps is None else 1, float(head_norm_eps or 0.0), float(post_mult), _stream()), "rows_attention")
+
+
+# ---------------------------------------------------------------------------------------------
+class StreamImage:
+    """The residual stream as it stands, in the activation type: what a block whose sublayers read
+    the stream itself hands on instead of a pending branch output (nothing is left to add)."""
+
+    __slots__ = ("image",)
+
+    def __init__(self, image) -> None:
+        self.image = image
+
+
+def branch_norm_add(resid, branch, weight, weight_offset: float, eps: float, scale: float, image=None):
+    """resid += scale * branch / sqrt(mean(branch^2) + eps) * (weight_offset + weight), float32
+    inside; ``image`` ([T, H] in the activation type, or None) receives the stream after that.
+    ``branch`` None: nothing is added (the image alone is made)."""
+    _gpu(resid, branch, weight, image)
+    T, H = resid.shape
+    _need(resid.dtype == torch.float32, "the residual stream is float32")
+    act = branch if branch is not None else image
+    _need(act is not None, "a branch or an image, or both")
+    if branch is not None:
+        _need(tuple(branch.shape) == (T, H), "the branch must be [T, H]")
+        _need(weight is not None and weight.numel() == H, "the norm's weight must have the row's size")
+    if image is not None:
+        _need(tuple(image.shape) == (T, H) and image.dtype == act.dtype, "the image must be [T, H] in the activation type")
+    _check(_load("rowwise").cw_branch_norm_add(_ptr(resid), _ptr(branch), _ptr(weight),
+                                               dtype_code(weight.dtype) if weight is not None else 0, float(weight_offset),
+                                               float(eps), float(scale), _ptr(image), dtype_code(act.dtype), T, H, _stream()),
+           "branch_norm_add")
+    return image
+
+
+def stream_norm(resid, weight, weight_offset: float, eps: float, out, rows=None) -> torch.Tensor:
+    """out[i] = resid[r] / sqrt(mean(resid[r]^2) + eps) * (weight_offset + weight), r = rows[i] (or i),
+    the product in float32 and rounded once; the stream is left as it is."""
+    _gpu(resid, weight, out, rows)
+    T, H = resid.shape
+    _need(resid.dtype == torch.float32, "the residual stream is float32")
+    n = T if rows is None else rows.numel()
+    if rows is not None:
+        _i32(rows, n, "rows")
+    _need(tuple(out.shape) == (n, H) and weight.numel() == H, f"out must be [{n}, {H}], the weight [{H}]")
+    _check(_load("rowwise").cw_stream_norm(_ptr(resid), _ptr(weight), dtype_code(weight.dtype), float(weight_offset), float(eps),
+                                           _ptr(out), dtype_code(out.dtype), _ptr(rows), n, H, _stream()), "stream_norm")
+    return out
+
+
+def headnorm_rope_store(proj: torch.Tensor, q_off: int, k_off: int, v_off: int, n_q_vectors: int, n_k_vectors: int, dim: int,
+                        nv: int, bias, q_weight, k_weight, eps: float, positions, freq, rot_dims: int, slots, k_plane,
+                        v_plane, values_from_keys: bool = False) -> None:
+    """Rows of ``proj`` [T, width] hold a token's query vectors (``n_q_vectors`` of ``dim`` elements
+    from column q_off), key vectors (``n_k_vectors`` from k_off) and value projection (``nv``
+    elements from v_off). ``bias`` ([width] or None) is added; every query and key vector by itself
+    is divided by its root mean square and multiplied by ``q_weight`` / ``k_weight`` ([dim], both or
+    neither), its first ``rot_dims`` elements rotated by the token's position (half-split pairs,
+    angle = position * freq[i], ``freq`` float32 [rot_dims / 2]). Queries are rewritten in place,
+    keys go to ``k_plane[slots[t]]``, values to ``v_plane[slots[t]]``: the biased value projection,
+    or with ``values_from_keys`` the biased key projection before norm and rotation. ``slots``
+    None or a negative slot: no cache row is written."""
+    _gpu(proj, bias, q_weight, k_weight, positions, freq, slots, k_plane, v_plane)
+    T, width = proj.shape
+    if positions is not None:
+        _i32(positions, T, "positions")
+    if slots is not None:
+        _i32(slots, T, "slots")
+    _need(bias is None or bias.numel() == width, "the bias must have one element per column of the projection")
+    _need((q_weight is None) == (k_weight is None), "norm weights for queries and keys, or for neither")
+    if q_weight is not None:
+        _need(q_weight.numel() == dim and k_weight.numel() == dim and q_weight.dtype == k_weight.dtype, "norm weights must be [dim]")
+    _need(rot_dims == 0 or (freq is not None and positions is not None and freq.dtype == torch.float32
+                            and freq.numel() >= rot_dims // 2), "freq must be float32 with rot_dims / 2 elements")
+    rows = 0
+    if slots is not None:
+        nk = n_k_vectors * dim
+        _need(k_plane is not None and k_plane.dtype == proj.dtype and k_plane.numel() % nk == 0, "the key plane must hold rows of the keys' width")
+        rows = k_plane.numel() // nk
+        _need(nv == 0 or (v_plane is not None and v_plane.dtype == proj.dtype and v_plane.numel() == rows * nv),
+              "key and value planes must hold the same number of rows")
+    _check(_load("rowwise").cw_headnorm_rope_store(
+        _ptr(proj), dtype_code(proj.dtype), width, int(q_off), int(k_off), int(v_off), int(n_q_vectors), int(n_k_vectors), int(dim),
+        int(nv), _ptr(bias), dtype_code(bias.dtype) if bias is not None else 0, _ptr(q_weight), _ptr(k_weight),
+        dtype_code(q_weight.dtype) if q_weight is not None else 0, float(eps), _ptr(positions), _ptr(freq), int(rot_dims),
+        _ptr(slots), _ptr(k_plane), _ptr(v_plane), int(bool(values_from_keys)), rows, T, _stream()), "headnorm_rope_store")
+
+
+def relu_squared_(x: torch.Tensor) -> torch.Tensor:
+    """x <- max(x, 0)^2, in place."""
+    _gpu(x)
+    _check(_load("rowwise").cw_relu_squared(_ptr(x), dtype_code(x.dtype), x.numel(), _stream()), "relu_squared")
+    return x
+
+
+def linear_relu_squared(x: torch.Tensor, weight: torch.Tensor, policy: "ProductPolicy | None" = None) -> torch.Tensor:
+    """max(x @ weight.T, 0)^2: the product, then the activation in place."""
+    return relu_squared_(linear(x, weight, policy=policy))
+
+
+def scale_(x: torch.Tensor, s: float) -> torch.Tensor:
+    """x <- s * x, in place on float32 (logits)."""
+    _gpu(x)
+    _need(x.dtype == torch.float32, "scale_ takes float32")
+    _check(_load("rowwise").cw_scale(_ptr(x), x.numel(), float(s), _stream()), "scale")
+    return x
+
+
+# ---------------------------------------------------------------------------------------------
+ROUTER_KINDS = {"sigmoid": 0, "softmax": 1}
+
+
+def moe_route(x: torch.Tensor, router: torch.Tensor, top: int, kind: str = "sigmoid", renormalize: bool = False):
+    """(choice int32 [T, top], score float32 [T, top]): the ``top`` experts with the largest
+    logistic (or softmax) of router x, the lower index first among equals, in falling order;
+    ``renormalize``: the chosen scores are divided by their sum. float32 sums."""
+    _gpu(x, router)
+    T, H = x.shape
+    E = router.shape[0]
+    _need(router.dim() == 2 and router.shape[1] == H and router.dtype == x.dtype, "the router must be [experts, H] in x's type")
+    _need(1 <= top <= E and kind in ROUTER_KINDS, f"top {top} of {E} experts, router kind {kind!r}")
+    choice = torch.empty((T, top), dtype=torch.int32, device=x.device)
+    score = torch.empty((T, top), dtype=torch.float32, device=x.device)
+    _check(_load("moe").cw_moe_route(_ptr(x), _ptr(router), dtype_code(x.dtype), T, H, E, top, ROUTER_KINDS[kind],
+                                     int(bool(renormalize)), _ptr(choice), _ptr(score), _stream()), "moe_route")
+    return choice, score
+
+
+class ExpertRows:
+    """The (token, choice) pairs of a step sorted by expert (``moe_plan``): ``row_pair`` int32
+    [max_rows] (pair index or -1), ``tile_expert`` int32 [max_tiles], ``n_tiles`` int32 [1], all on
+    the device; every tile of ``tile_rows`` rows belongs to one expert."""
+
+    __slots__ = ("row_pair", "tile_expert", "n_tiles", "max_tiles", "max_rows", "n_pairs")
+
+
+def moe_plan(choice: torch.Tensor, experts: int) -> ExpertRows:
+    _gpu(choice)
+    _need(choice.dtype == torch.int32, "choices are int32")
+    lib = _load("moe")
+    plan = ExpertRows()
+    plan.n_pairs = choice.numel()
+    plan.max_tiles = int(lib.cw_moe_max_tiles(plan.n_pairs, experts))
+    plan.max_rows = plan.max_tiles * int(lib.cw_moe_tile_rows())
+    plan.row_pair = torch.empty(max(plan.max_rows, 1), dtype=torch.int32, device=choice.device)
+    plan.tile_expert = torch.empty(max(plan.max_tiles, 1), dtype=torch.int32, device=choice.device)
+    plan.n_tiles = torch.empty(1, dtype=torch.int32, device=choice.device)
+    _check(lib.cw_moe_plan(_ptr(choice), plan.n_pairs, experts, _ptr(plan.row_pair), plan.max_rows, _ptr(plan.tile_expert),
+                           plan.max_tiles, _ptr(plan.n_tiles), _stream()), "moe_plan")
+    return plan
+
+
+def moe_gate_up(x: torch.Tensor, gate_up: torch.Tensor, plan: ExpertRows, score: torch.Tensor, top: int,
+                scale_input: bool) -> torch.Tensor:
+    """inner [max_rows, ff] = silu(gate_e u) * (up_e u) for every row of the plan, u the row's token
+    of ``x`` [T, H] (times the pair's score, rounded to x's type, with ``scale_input``); ``gate_up``
+    [experts, 2 * ff, H], gate rows first. Rows that hold no pair are zero."""
+    _gpu(x, gate_up, score)
+    T, H = x.shape
+    _need(gate_up.dim() == 3 and gate_up.shape[2] == H and gate_up.shape[1] % 2 == 0 and gate_up.dtype == x.dtype,
+          "gate_up must be [experts, 2 * ff, H] in x's type")
+    _need(plan.n_pairs == T * top and score.numel() == T * top and score.dtype == torch.float32, "one score a pair")
+    ff = gate_up.shape[1] // 2
+    inner = torch.empty((max(plan.max_rows, 1), ff), dtype=x.dtype, device=x.device)
+    _check(_load("moe").cw_moe_expert_product(0, _ptr(x), _ptr(gate_up), _ptr(inner), dtype_code(x.dtype), _ptr(plan.row_pair),
+                                              _ptr(plan.tile_expert), _ptr(plan.n_tiles), plan.max_tiles, _ptr(score), top, H, ff,
+                                              int(bool(scale_input)), _stream()), "moe_gate_up")
+    return inner
+
+
+def moe_down(inner: torch.Tensor, down: torch.Tensor, plan: ExpertRows, score: torch.Tensor, top: int, scale_output: bool,
+             out: torch.Tensor) -> torch.Tensor:
+    """out[pair] = down_e inner[row] for every row that holds a pair (times the pair's score with
+    ``scale_output``); ``down`` [experts, H, ff], ``out`` [pairs, H]."""
+    _gpu(inner, down, score, out)
+    ff = inner.shape[1]
+    _need(down.dim() == 3 and down.shape[2] == ff and down.dtype == inner.dtype, "down must be [experts, H, ff] in the rows' type")
+    H = down.shape[1]
+    _need(inner.shape[0] >= plan.max_rows and tuple(out.shape) == (plan.n_pairs, H) and out.dtype == inner.dtype, "out must be [pairs, H]")
+    _check(_load("moe").cw_moe_expert_product(1, _ptr(inner), _ptr(down), _ptr(out), dtype_code(inner.dtype), _ptr(plan.row_pair),
+                                              _ptr(plan.tile_expert), _ptr(plan.n_tiles), plan.max_tiles, _ptr(score), top, ff, H,
+                                              int(bool(scale_output)), _stream()), "moe_down")
+    return out
+
+
+def moe_combine(y: torch.Tensor, top: int, out: torch.Tensor) -> torch.Tensor:
+    """out[t] = y[t * top] + ... + y[t * top + top - 1], added in that order in float32."""
+    _gpu(y, out)
+    T, H = out.shape
+    _need(tuple(y.shape) == (T * top, H) and y.dtype == out.dtype, "y must be [T * top, H]")
+    _check(_load("moe").cw_moe_combine(_ptr(y), _ptr(out), dtype_code(out.dtype), T, top, H, _stream()), "moe_combine")
+    return out

@@ -118,3 +118,43 @@ class ParallelBlock:
             return pending
         ops.gated_residual_add(resid, pending)
         return None
+
+
+class BranchNormBlock:
+    """x = x + c * N1(mixer(x)); x = x + c * N2(ffn(x)): mixer and feed-forward read the stream
+    itself, and what is normed is their output (``BranchRMSNorm``, whose spec holds c). The
+    feed-forward and its norm may be absent.
+
+    The stream is float32; the sublayers read its image in the activation type, which the kernel
+    that adds a normed branch writes beside the stream. So the block has nothing pending when it
+    is done: it hands on the image (``ops.StreamImage``), which the next block of this kind reads
+    instead of making it again."""
+
+    def __init__(self, mixer, mixer_norm, feed_forward=None, ffn_norm=None) -> None:
+        if (feed_forward is None) != (ffn_norm is None):
+            raise ValueError("a block has a feed-forward and its norm, or neither")
+        for norm in (mixer_norm, ffn_norm):
+            if norm is not None and not (hasattr(norm, "join") and hasattr(norm, "image")):
+                raise TypeError("the norms of a 'branchnorm' block norm a branch as it joins the stream (join / image)")
+        self.mixer, self.mixer_norm, self.feed_forward, self.ffn_norm = mixer, mixer_norm, feed_forward, ffn_norm
+
+    def parts(self) -> dict:
+        parts = {"mixer": self.mixer}
+        if self.feed_forward is not None:
+            parts["feed_forward"] = self.feed_forward
+        parts["mixer_norm"] = self.mixer_norm
+        if self.ffn_norm is not None:
+            parts["ffn_norm"] = self.ffn_norm
+        return parts
+
+    def forward(self, resid, delta, ctx, cache):
+        if isinstance(delta, ops.StreamImage):
+            x = delta.image
+        elif delta is None:
+            x = self.mixer_norm.image(resid)
+        else:
+            raise TypeError("a 'branchnorm' block cannot add the pending output of a block of another kind")
+        x = self.mixer_norm.join(resid, self.mixer.forward(x, ctx, cache))
+        if self.feed_forward is not None:
+            x = self.ffn_norm.join(resid, self.feed_forward.forward(x, ctx))
+        return ops.StreamImage(x)

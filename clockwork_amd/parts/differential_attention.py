@@ -1,7 +1,9 @@
 """Attention with two score maps a head over shared values (``DifferentialAttentionSpec``).
 
 Steps: one fused q/k/v product; one kernel adds the biases, rewrites the queries and writes keys
-and values to their pages (every token of the step is cached before any query reads); the
+and values to their pages (every token of the step is cached before any query reads; with
+``qk_norm`` or a position encoding the same kernel norms every query and key vector, each map of
+each head by itself, and rotates it by the token's position); the
 attention kernel runs both maps of a head in one workgroup, subtracts the second from the first
 with the layer's lambda, norms the head's output and scales it; output product. Keys
 [kv_heads, 2, key_dim] and values [kv_heads, value_dim] are two planes of a ``PagedRowsSpec``;
@@ -39,6 +41,11 @@ class DifferentialAttention(Part):
         }
         if s.qkv_bias:
             specs["qkv_bias"] = ParamSpec((width,), precision="stored", init=("normal", 0.02))
+        if s.out_bias:
+            specs["out_bias"] = ParamSpec((s.hidden_size,), precision="compute", init=("normal", 0.02))
+        if s.qk_norm:
+            specs["q_norm"] = ParamSpec((s.key_dim,), precision="stored", init=("one_plus_uniform", 0.3))
+            specs["k_norm"] = ParamSpec((s.key_dim,), precision="stored", init=("one_plus_uniform", 0.3))
         for name in ("lq1", "lk1", "lq2", "lk2"):
             specs[name] = ParamSpec((s.key_dim,), precision="float32", init=("normal", 0.1))
         return specs
@@ -60,7 +67,15 @@ class DifferentialAttention(Part):
     def bind(self, params, device, dtype) -> None:
         s = self.spec
         self.qkv_weight, self.qkv_bias = params["qkv_weight"], params.get("qkv_bias")
-        self.out_weight = params["out_weight"]
+        self.out_weight, self.out_bias = params["out_weight"], params.get("out_bias")
+        self.q_norm, self.k_norm = params.get("q_norm"), params.get("k_norm")
+        # rotation frequencies base^(-2i / n), made on the host in float64 and rounded once
+        self.rot_dims = s.position.rotary_dim if s.position is not None else 0
+        self.freq = None
+        if self.rot_dims:
+            freq = torch.tensor([float(s.position.theta) ** (-2.0 * i / self.rot_dims) for i in range(self.rot_dims // 2)],
+                                dtype=torch.float64)
+            self.freq = freq.to(torch.float32).to(device)
         # lambda = exp(lq1 . lk1) - exp(lq2 . lk2) + lambda_init: one float32 number a layer
         lam = (torch.exp((params["lq1"].float() * params["lk1"].float()).sum())
                - torch.exp((params["lq2"].float() * params["lk2"].float()).sum()) + s.lambda_init)
@@ -98,8 +113,13 @@ class DifferentialAttention(Part):
             raise NotImplementedError("this mixer writes its own keys and values: it cannot borrow another entry's cache")
         k_plane, v_plane = cache.planes["k"], cache.planes["v"]
         qkv = ops.linear(x, self.qkv_weight, policy=policy)
-        ops.bias_store(qkv, 0, self.q_width, self.q_width + self.k_width, self.q_width, self.k_width, self.v_width,
-                       self.qkv_bias, ctx.slots[cache.group], k_plane, v_plane)
+        if s.qk_norm or self.rot_dims:
+            ops.headnorm_rope_store(qkv, 0, self.q_width, self.q_width + self.k_width, s.num_heads * MAPS, s.num_kv_heads * MAPS,
+                                    s.key_dim, self.v_width, self.qkv_bias, self.q_norm, self.k_norm, s.norm_eps, ctx.positions,
+                                    self.freq, self.rot_dims, ctx.slots[cache.group], k_plane, v_plane)
+        else:
+            ops.bias_store(qkv, 0, self.q_width, self.q_width + self.k_width, self.q_width, self.k_width, self.v_width,
+                           self.qkv_bias, ctx.slots[cache.group], k_plane, v_plane)
         out = torch.empty((x.shape[0], s.num_heads * s.value_dim), dtype=x.dtype, device=x.device)
         items, n_items, runs = self._plan(ctx)
         kind, size = self.mask()
@@ -107,4 +127,4 @@ class DifferentialAttention(Part):
                            ctx.block_tables[cache.group], ctx.ctx_lens, ctx.cu_q, items, n_items, s.num_heads, s.num_kv_heads,
                            s.key_dim, s.value_dim, cache.block_size, s.scale, maps=MAPS, mask=kind, mask_size=size, lam=self.lam,
                            head_norm_eps=s.norm_eps, post_mult=1.0 - s.lambda_init, mfma=self.mfma, key_runs=runs)
-        return ops.linear(out, self.out_weight, policy=policy)
+        return ops.linear(out, self.out_weight, self.out_bias, policy=policy)

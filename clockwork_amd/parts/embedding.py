@@ -114,9 +114,11 @@ class LinearHead(Part):
 
     def forward(self, rows: torch.Tensor, ctx) -> torch.Tensor:
         logits = ops.linear(rows, self.weight, out_dtype=torch.float32, policy=getattr(ctx, "products", None))
+        if self.spec.scale is not None:
+            ops.scale_(logits, self.spec.scale)
         if self.spec.softcap is not None:
             ops.softcap_(logits, self.spec.softcap)
         return logits
 
     def kernel_libraries(self) -> list:
-        return [("rowwise", None)] if self.spec.softcap is not None else []
+        return [("rowwise", None)] if self.spec.softcap is not None or self.spec.scale is not None else []

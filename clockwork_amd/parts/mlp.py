@@ -68,8 +68,9 @@ class GatedMLP(Part):
 
 
 class DenseMLP(Part):
-    """down(gelu(up(x))) (``DenseMLPSpec``): the up product with the erf GELU (float32 inside) in
-    its epilogue for few rows, as a kernel of its own behind the product otherwise; the down product."""
+    """down(act(up(x))) (``DenseMLPSpec``). "gelu": the up product with the erf GELU (float32
+    inside) in its epilogue for few rows, as a kernel of its own behind the product otherwise;
+    "relu2": the product, then max(z, 0)^2 in place; the down product."""
 
     graph_safe = True
 
@@ -89,4 +90,6 @@ class DenseMLP(Part):
 
     def forward(self, x, ctx) -> torch.Tensor:
         policy = getattr(ctx, "products", None)
+        if self.spec.activation == "relu2":
+            return ops.linear(ops.linear_relu_squared(x, self.up, policy=policy), self.down, policy=policy)
         return ops.linear(ops.linear_gelu(x, self.up, policy=policy), self.down, policy=policy)

@@ -108,3 +108,48 @@ class DynamicTanh(Part):
         n = resid.shape[0] if rows is None else rows.numel()
         out = torch.empty((n, self.spec.size), dtype=self.dtype, device=resid.device)
         return ops.add_dynamic_tanh(resid, delta, self.spec.delta_scale, extra, self.weight, self.bias, self.alpha, out, rows)
+
+
+class BranchRMSNorm(Part):
+    """RMS norm with a weight kept as a distance from a constant (``BranchRMSNormSpec``), float32
+    throughout. ``join(resid, branch, image)`` norms a sublayer's output, adds it to the stream
+    multiplied by the spec's ``branch_scale`` and leaves the stream's image in the activation type,
+    all in one kernel; ``forward(resid, delta, rows)`` is the norm of the stream itself (a final
+    norm): nothing may be pending then but an ``ops.StreamImage``, which says so."""
+
+    graph_safe = True
+
+    def __init__(self, spec) -> None:
+        self.spec = spec
+
+    def param_specs(self):
+        return {"weight": ParamSpec((self.spec.size,), precision="stored", init=("normal", 0.1))}
+
+    def kernel_libraries(self) -> list:
+        return [("rowwise", None)]
+
+    def bind(self, params, device, dtype) -> None:
+        self.weight = params["weight"]
+        self.dtype = dtype
+
+    def image(self, resid: torch.Tensor) -> torch.Tensor:
+        """The stream in the activation type (the stream itself where that is float32)."""
+        if self.dtype == torch.float32:
+            return resid
+        return ops.branch_norm_add(resid, None, None, 0.0, self.spec.eps, 0.0, torch.empty(tuple(resid.shape), dtype=self.dtype, device=resid.device))
+
+    def join(self, resid: torch.Tensor, branch) -> torch.Tensor:
+        """resid += branch_scale * N(branch); returns the stream's image in the activation type."""
+        s = self.spec
+        if isinstance(branch, ops.PartialSums):
+            branch = branch.sum(self.dtype)
+        image = None if self.dtype == torch.float32 else torch.empty(tuple(resid.shape), dtype=self.dtype, device=resid.device)
+        ops.branch_norm_add(resid, branch, self.weight, s.weight_offset, s.eps, s.branch_scale, image)
+        return resid if image is None else image
+
+    def forward(self, resid: torch.Tensor, delta, rows=None) -> torch.Tensor:
+        if delta is not None and not isinstance(delta, ops.StreamImage):
+            raise TypeError("this norm reads the stream as it stands: a pending branch output must have joined it before")
+        n = resid.shape[0] if rows is None else rows.numel()
+        out = torch.empty((n, self.spec.size), dtype=self.dtype, device=resid.device)
+        return ops.stream_norm(resid, self.weight, self.spec.weight_offset, self.spec.eps, out, rows)

@@ -78,12 +78,14 @@ class TokenEmbeddingSpec:
 class LinearHeadSpec:
     """logits = rows @ W^T with W [vocab, hidden], no bias, float32 logits. ``tied``: W is the
     embedding's table (one buffer, two uses) unless the checkpoint brings a head of its own.
-    ``softcap`` c: the logits are capped, c * tanh(logits / c)."""
+    ``softcap`` c: the logits are capped, c * tanh(logits / c). ``scale`` s: the logits are
+    multiplied by s (before a cap)."""
 
     vocab_size: int
     hidden_size: int
     tied: bool = False
     softcap: Optional[float] = None  # logits <- softcap * tanh(logits / softcap)
+    scale: Optional[float] = None    # logits <- scale * logits
 
 
 @dataclass(frozen=True)
@@ -216,15 +218,16 @@ class DynamicTanhSpec:
 
 @dataclass(frozen=True)
 class DenseMLPSpec:
-    """down(act(up(x))), no gate, no biases; ``activation`` "gelu" (the erf form)."""
+    """down(act(up(x))), no gate, no biases; ``activation`` "gelu" (the erf form) or "relu2"
+    (max(z, 0)^2)."""
 
     hidden_size: int
     intermediate_size: int
     activation: str = "gelu"
 
     def __post_init__(self):
-        if self.activation not in ("gelu",):
-            raise ValueError(f"activation {self.activation!r}: expected 'gelu'")
+        if self.activation not in ("gelu", "relu2"):
+            raise ValueError(f"activation {self.activation!r}: expected 'gelu' or 'relu2'")
 
 
 @dataclass(frozen=True)
@@ -234,7 +237,14 @@ class DifferentialAttentionSpec:
     all from biased projections (``qkv_bias``). The head's output is A_1 - lambda * A_2 with
     lambda = exp(lq1 . lk1) - exp(lq2 . lk2) + ``lambda_init`` (four learned vectors of key_dim, one
     number a layer), then divided by its root mean square over value_dim (``norm_eps`` inside the
-    root, no weight) and multiplied by 1 - ``lambda_init``. No position encoding.
+    root, no weight) and multiplied by 1 - ``lambda_init``.
+
+    ``qk_norm``: every query and key vector of key_dim elements (each map of each head by itself)
+    is divided by its root mean square (``norm_eps``) and multiplied by a weight of key_dim
+    elements, one for all query vectors and one for all key vectors, after the bias and before the
+    rotation. ``position``: a ``RopeNeoxSpec``, applied to every query and key vector by itself
+    (its first ``rotary_dim`` elements); None: no position encoding. ``out_bias``: the output
+    projection has a bias.
 
     What a token sees: ``segment`` S: the earlier tokens of its own run of S positions (runs
     counted from position 0); ``window`` W: itself and the W - 1 before it; neither: all earlier ones."""
@@ -250,12 +260,17 @@ class DifferentialAttentionSpec:
     segment: Optional[int] = None
     window: Optional[int] = None
     qkv_bias: bool = True
+    qk_norm: bool = False
+    position: Any = None
+    out_bias: bool = False
 
     def __post_init__(self):
         if self.num_heads < 1 or self.num_kv_heads < 1 or self.num_heads % self.num_kv_heads:
             raise ValueError(f"num_heads {self.num_heads} is not a multiple of num_kv_heads {self.num_kv_heads}")
         if self.key_dim < 1 or self.value_dim < 1:
             raise ValueError("key_dim and value_dim must be positive")
+        if self.position is not None and not 0 <= self.position.rotary_dim <= self.key_dim:
+            raise ValueError(f"rotary_dim {self.position.rotary_dim} exceeds key_dim {self.key_dim}")
         if self.segment is not None and self.window is not None:
             raise ValueError("an attention mask has segments or a window, not both")
         for name in ("segment", "window"):
@@ -297,3 +312,93 @@ class LatentAttentionSpec:
             raise ValueError(f"rotary_dims {self.rotary_dims} must be even and at most rope_dim {self.rope_dim}")
         if self.window is not None and self.window < 1:
             raise ValueError(f"window must be positive, got {self.window}")
+
+
+@dataclass(frozen=True)
+class BranchRMSNormSpec:
+    """An RMS norm whose weight is kept as its distance from ``weight_offset``:
+    N(y) = y / sqrt(mean(y^2) + eps) * (weight_offset + w), float32 throughout. It has two uses.
+    On a branch: a sublayer's OUTPUT is normed and joins the float32 stream multiplied by
+    ``branch_scale``, x <- x + branch_scale * N(branch) (the "branchnorm" block arrangement, whose
+    sublayers read the stream itself). On the stream: N(x) of chosen rows (a model's final norm)."""
+
+    size: int
+    eps: float
+    branch_scale: float = 1.0
+    weight_offset: float = 1.0
+
+
+@dataclass(frozen=True)
+class GatedAttentionSpec:
+    """Grouped softmax attention over paged key rows [kv_heads, key_dim] and value rows
+    [kv_heads, value_dim], with options that plain attention has not:
+
+    * ``qk_norm``: every head's query and key vector is divided by its root mean square
+      (``norm_eps`` inside the root) and multiplied by a weight of key_dim elements (one for all
+      query heads, one for all key heads), before the rotation.
+    * ``position``: a ``RopeNeoxSpec`` (the first ``rotary_dim`` elements of every head's query
+      and key are rotated) or None.
+    * ``values``: "projection" (a value projection of its own) or "keys": the values are the key
+      projections as they leave the product, before norm and rotation (value_dim == key_dim, no
+      value matrix).
+    * ``output_gate``: the concatenated heads are multiplied by the logistic function of one more
+      projection of the mixer's input before the output projection.
+    * ``window`` W: a token sees itself and the W - 1 tokens before it; None: all of them.
+    * ``qkv_bias`` / ``out_bias``."""
+
+    hidden_size: int
+    num_heads: int
+    num_kv_heads: int
+    key_dim: int
+    value_dim: int
+    scale: float
+    norm_eps: float = 1e-6
+    window: Optional[int] = None
+    qk_norm: bool = True
+    position: Any = None
+    values: str = "projection"
+    output_gate: bool = False
+    qkv_bias: bool = False
+    out_bias: bool = False
+
+    def __post_init__(self):
+        if self.num_heads < 1 or self.num_kv_heads < 1 or self.num_heads % self.num_kv_heads:
+            raise ValueError(f"num_heads {self.num_heads} is not a multiple of num_kv_heads {self.num_kv_heads}")
+        if self.key_dim < 1 or self.value_dim < 1:
+            raise ValueError("key_dim and value_dim must be positive")
+        if self.values not in ("projection", "keys"):
+            raise ValueError(f"values {self.values!r}: expected 'projection' or 'keys'")
+        if self.values == "keys" and self.value_dim != self.key_dim:
+            raise ValueError(f"values that are the keys have the keys' size: value_dim {self.value_dim} != key_dim {self.key_dim}")
+        if self.position is not None and not 0 <= self.position.rotary_dim <= self.key_dim:
+            raise ValueError(f"rotary_dim {self.position.rotary_dim} exceeds key_dim {self.key_dim}")
+        if self.window is not None and self.window < 1:
+            raise ValueError(f"window must be positive, got {self.window}")
+
+
+@dataclass(frozen=True)
+class RoutedExpertsSpec:
+    """A feed-forward made of ``num_experts`` small gated ones, E(u) = down(silu(gate u) * (up u)),
+    no biases, of which every token uses ``top_k``: r = ``router``(W_r x) in float32 ("sigmoid":
+    the logistic function of each logit by itself; "softmax": over the experts), the top_k
+    largest r chosen (the lower index first among equals), divided by their sum if
+    ``renormalize``. ``weight_on`` "input": the result is the sum of E_e(r_e x); "output": the sum
+    of r_e E_e(x)."""
+
+    hidden_size: int
+    intermediate_size: int
+    num_experts: int
+    top_k: int
+    router: str = "sigmoid"
+    renormalize: bool = False
+    weight_on: str = "input"
+
+    def __post_init__(self):
+        if min(self.hidden_size, self.intermediate_size, self.num_experts) < 1:
+            raise ValueError("hidden_size, intermediate_size and num_experts must be positive")
+        if not 1 <= self.top_k <= self.num_experts:
+            raise ValueError(f"top_k {self.top_k} must be between 1 and num_experts {self.num_experts}")
+        if self.router not in ("sigmoid", "softmax"):
+            raise ValueError(f"router {self.router!r}: expected 'sigmoid' or 'softmax'")
+        if self.weight_on not in ("input", "output"):
+            raise ValueError(f"weight_on {self.weight_on!r}: expected 'input' or 'output'")

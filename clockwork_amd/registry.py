@@ -40,6 +40,7 @@ _BUILTIN_ARCHITECTURES = {
     "qwen2": "clockwork_amd.models.qwen2",
     "Fuvavik": "clockwork_amd.models.fuvavik",
     "Pesorax": "clockwork_amd.models.pesorax",
+    "Nenodra": "clockwork_amd.models.nenodra",
 }
 
 
@@ -103,10 +104,14 @@ _BUILTIN_PARTS = {
     "DenseMLPSpec": ("clockwork_amd.parts.mlp", "DenseMLP"),
     "DifferentialAttentionSpec": ("clockwork_amd.parts.differential_attention", "DifferentialAttention"),
     "LatentAttentionSpec": ("clockwork_amd.parts.latent_attention", "LatentAttention"),
+    "BranchRMSNormSpec": ("clockwork_amd.parts.norm", "BranchRMSNorm"),
+    "GatedAttentionSpec": ("clockwork_amd.parts.gated_attention", "GatedAttention"),
+    "RoutedExpertsSpec": ("clockwork_amd.parts.moe", "RoutedExperts"),
 }
 _ARRANGEMENTS: dict[str, Callable[..., Any]] = {}
 _BUILTIN_ARRANGEMENTS = {"prenorm": ("clockwork_amd.parts.block", "PreNormBlock"),
-                         "parallel": ("clockwork_amd.parts.block", "ParallelBlock")}
+                         "parallel": ("clockwork_amd.parts.block", "ParallelBlock"),
+                         "branchnorm": ("clockwork_amd.parts.block", "BranchNormBlock")}
 
 
 def register_part(spec_type: type, factory: Callable[[Any], Any]) -> None:
