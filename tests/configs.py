@@ -201,3 +201,74 @@ PESORAX_LONG = {
 }
 # name -> (config, weight seed, cache block size)
 PESORAX_CONFIGS = {"PA": (PESORAX_A, 31, 8), "PB": (PESORAX_B, 32, 16), "PC": (PESORAX_C, 33, 4)}
+
+
+# ---- Nenodra: small models that differ in every size and constant; layers of one model differ too.
+def _nenodra_mlp(mlp):
+    if mlp is None or isinstance(mlp, dict):
+        return mlp
+    if isinstance(mlp, int):
+        return {"kind": "dense", "ff": mlp}
+    ff, experts, top = mlp
+    return {"kind": "moe", "expert": {"ff": ff}, "router": {"experts": experts, "top": top}}
+
+
+def _nenodra_two_map(heads, kv_heads, dim, vdim, scale, diff, window, base, rot_dims, mlp):
+    return {"type": "attention",
+            "mixer": {"heads": heads, "kv_heads": kv_heads, "dim": dim, "vdim": vdim, "scale": scale, "diff": diff,
+                      "mask": {"size": window}, "rot": {"base": base, "dims": rot_dims}},
+            "mlp": _nenodra_mlp(mlp)}
+
+
+def _nenodra_gated(heads, kv_heads, dim, scale, window, base, rot_dims, mlp):
+    return {"type": "attention_2",
+            "mixer": {"heads": heads, "kv_heads": kv_heads, "dim": dim, "vdim": dim, "scale": scale,
+                      "mask": {"size": window}, "rot": {"base": base, "dims": rot_dims}},
+            "mlp": _nenodra_mlp(mlp)}
+
+
+# four layers that share nothing: three query heads a key/value head, windows of 9, 33, 5 and 17,
+# rotations of a part of the vector and of all of it, two and three experts a token (all of three),
+# a layer without a feed-forward; the three model-wide constants all differ
+NENODRA_A = {
+    "architecture": "Nenodra", "vocab": 300, "width": 96, "residual_mult": 0.7, "logit_scale": 1.3, "norm": {"eps": 1e-5},
+    "layers": [
+        _nenodra_gated(6, 2, 16, 0.2, 9, 100.0, 8, (40, 5, 2)),
+        _nenodra_two_map(4, 2, 8, 24, 0.3, 0.3, 33, 1000.0, 8, 72),
+        _nenodra_two_map(2, 2, 24, 8, 0.25, 0.8, 5, 50.0, 12, (24, 3, 3)),
+        _nenodra_gated(3, 1, 40, 0.16, 17, 10000.0, 40, None),
+    ],
+}
+# a width that is no multiple of 8, a window longer than any request of the tests (every earlier key
+# is seen) and one of 1 (a token sees itself alone), no rotation at all in one layer, one expert of
+# two, constants of 1
+NENODRA_B = {
+    "architecture": "Nenodra", "vocab": 127, "width": 100, "residual_mult": 1.0, "logit_scale": 1.0, "norm": {"eps": 3e-4},
+    "layers": [
+        _nenodra_two_map(3, 1, 40, 24, 0.16, 0.5, 300, 250000.0, 2, (50, 2, 1)),
+        _nenodra_gated(5, 5, 12, 0.3, 1, 50.0, 12, 130),
+        _nenodra_two_map(2, 1, 8, 32, 0.35, 0.1, 40, 10.0, 0, (36, 7, 4)),
+    ],
+}
+# one head everywhere, sizes of 1 and 2 where the design allows them, a single expert
+NENODRA_C = {
+    "architecture": "Nenodra", "vocab": 64, "width": 48, "residual_mult": 0.25, "logit_scale": 0.1, "norm": {"eps": 1e-6},
+    "layers": [
+        _nenodra_gated(1, 1, 2, 0.5, 16, 4.0, 2, (1, 1, 1)),
+        _nenodra_two_map(1, 1, 32, 1, 0.18, 0.6, 17, 500.0, 16, 24),
+    ],
+}
+# layers of unlike sizes for long requests: windows of 77 to 1500, head sizes that the matrix cores
+# take and ones that they do not, sixteen experts of which a token uses four
+NENODRA_LONG = {
+    "architecture": "Nenodra", "vocab": 211, "width": 192, "residual_mult": 0.4, "logit_scale": 0.8, "norm": {"eps": 2e-6},
+    "layers": [
+        _nenodra_two_map(6, 3, 32, 48, 0.3, 0.4, 200, 10000.0, 32, 384),
+        _nenodra_gated(8, 2, 64, 0.2, 513, 10000.0, 32, (64, 16, 4)),
+        _nenodra_two_map(8, 2, 64, 128, 0.15, 0.7, 1500, 500000.0, 64, 100),
+        _nenodra_gated(4, 4, 128, 0.12, 77, 500.0, 128, None),
+        _nenodra_gated(6, 2, 24, 0.25, 130, 1000.0, 20, (40, 3, 2)),
+    ],
+}
+# name -> (config, weight seed, cache block size)
+NENODRA_CONFIGS = {"NA": (NENODRA_A, 41, 8), "NB": (NENODRA_B, 42, 16), "NC": (NENODRA_C, 43, 4)}
