@@ -2,7 +2,7 @@
 
     python bench.py [--gpus 1] [--steps K] [--warmup W] [--batch B] [--layers L] [--dtype bfloat16] [--shape 1.5b]
     python bench.py --workload mixed|arrivals|agent [--shape 7b] [--requests 64]
-    python bench.py --design fuvavik|pesorax [--size s|m|l] [--layers L] [--batch B]
+    python bench.py --design fuvavik|pesorax|nenodra [--size s|m|l] [--layers L] [--batch B]
 
 Default workload: the layer sizes of Qwen2.5-1.5B with random weights (seed 2), bfloat16,
 8 requests that each hold a 2048-token prompt, context limit 4096, pages of 16 tokens. A
@@ -557,7 +557,34 @@ def pesorax_config(size: dict, layers: int, max_positions: int) -> dict:
             "layers": [attention if i % 2 == 0 else latent for i in range(distinct)]}
 
 
-DESIGNS = {"fuvavik": (FUVAVIK_SIZES, fuvavik_config), "pesorax": (PESORAX_SIZES, pesorax_config)}
+# Layer sizes for ``--design nenodra``: the same widths, head counts and feed-forwards. The one-map
+# mixer has heads of the Qwen2 head's size (its values are its keys), the two-map mixer key rows
+# of 64 elements a map and values of that size; both behind a window of half the prompt. Dense
+# feed-forwards have the Qwen2 layer's inner width, routed ones eight experts of half that width
+# of which a token uses two (as many active parameters). Four layers, one of each combination.
+NENODRA_SIZES = {
+    "s": dict(width=896, heads=14, kv_heads=2, dim=64, vdim=64, head_dim=64, window=1024, ff=4864, experts=8, top=2, layers=4),
+    "m": dict(width=1536, heads=12, kv_heads=2, dim=64, vdim=128, head_dim=128, window=1024, ff=8960, experts=8, top=2, layers=4),
+    "l": dict(width=2048, heads=16, kv_heads=2, dim=64, vdim=128, head_dim=128, window=1024, ff=11008, experts=8, top=2, layers=4),
+}
+
+
+def nenodra_config(size: dict, layers: int, max_positions: int) -> dict:
+    dense = {"kind": "dense", "ff": size["ff"]}
+    routed = {"kind": "moe", "expert": {"ff": size["ff"] // size["top"]}, "router": {"experts": size["experts"], "top": size["top"]}}
+    rot = {"base": 10000.0, "dims": 64}
+    gated = {"heads": size["heads"], "kv_heads": size["kv_heads"], "dim": size["head_dim"], "vdim": size["head_dim"],
+             "scale": size["head_dim"] ** -0.5, "mask": {"size": size["window"]}, "rot": rot}
+    two_map = {"heads": size["heads"], "kv_heads": size["kv_heads"], "dim": size["dim"], "vdim": size["vdim"], "diff": 0.5,
+               "scale": size["dim"] ** -0.5, "mask": {"size": size["window"]}, "rot": rot}
+    kinds = [("attention_2", gated, dense), ("attention", two_map, routed), ("attention", two_map, dense), ("attention_2", gated, routed)]
+    return {"architecture": "Nenodra", "vocab": DESIGN_VOCAB, "width": size["width"], "residual_mult": 0.5, "logit_scale": 0.5,
+            "norm": {"eps": 1e-6},
+            "layers": [{"type": kinds[i % 4][0], "mixer": kinds[i % 4][1], "mlp": kinds[i % 4][2]} for i in range(layers)]}
+
+
+DESIGNS = {"fuvavik": (FUVAVIK_SIZES, fuvavik_config), "pesorax": (PESORAX_SIZES, pesorax_config),
+           "nenodra": (NENODRA_SIZES, nenodra_config)}
 
 
 def qwen2_config_like(size: dict, layers: int, max_positions: int) -> dict:
