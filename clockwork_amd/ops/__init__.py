@@ -139,11 +139,11 @@ def _declare(name: str, lib: ctypes.CDLL) -> None:
             "cw_scale": [P, L, F, P],
         },
         "moe": {
-            "cw_moe_tile_rows": [],
-            "cw_moe_max_tiles": [I, I],
+            "cw_moe_tile_rows": [I],
+            "cw_moe_max_tiles": [I, I, I],
             "cw_moe_route": [P, P, I, I, I, I, I, I, I, P, P, P],
-            "cw_moe_plan": [P, I, I, P, I, P, I, P, P],
-            "cw_moe_expert_product": [I, P, P, P, I, P, P, P, I, P, I, I, I, I, P],
+            "cw_moe_plan": [P, I, I, I, P, I, P, I, P, P],
+            "cw_moe_expert_product": [I, I, P, P, P, I, P, P, P, I, P, I, I, I, I, P],
             "cw_moe_combine": [P, P, I, I, I, I, P],
         },
         "rows_attention": {
@@ -1960,27 +1960,47 @@ def moe_route(x: torch.Tensor, router: torch.Tensor, top: int, kind: str = "sigm
     return choice, score
 
 
+MOE_KERNELS = {"plain": 0, "stream": 1, "wide": 2}
+# rows an expert from which a step's experts run on the wide tiles of the matrix-core kernel
+MOE_WIDE_FROM = 48
+
+
+def moe_kernel_for(dtype, n_pairs: int, experts: int, hidden: int, ff: int) -> str:
+    """Which kernel runs the experts' products of a step: by type, sizes and the step's shape alone
+    (never by what the router chose), so a captured step replays. bfloat16 with widths that are a
+    multiple of 8 runs on the matrix cores: "wide" tiles of 128 rows from ``MOE_WIDE_FROM`` rows an
+    expert on average, else "stream" (tiles of 16 rows, the expert's matrix read once a tile);
+    everything else, float32 included, "plain" arithmetic."""
+    if dtype != torch.bfloat16 or hidden % 8 or ff % 8:
+        return "plain"
+    return "wide" if n_pairs >= MOE_WIDE_FROM * experts else "stream"
+
+
 class ExpertRows:
     """The (token, choice) pairs of a step sorted by expert (``moe_plan``): ``row_pair`` int32
     [max_rows] (pair index or -1), ``tile_expert`` int32 [max_tiles], ``n_tiles`` int32 [1], all on
-    the device; every tile of ``tile_rows`` rows belongs to one expert."""
+    the device; every tile of ``tile_rows`` rows belongs to one expert. ``kernel`` names the kernel
+    whose tiles these are."""
 
-    __slots__ = ("row_pair", "tile_expert", "n_tiles", "max_tiles", "max_rows", "n_pairs")
+    __slots__ = ("row_pair", "tile_expert", "n_tiles", "max_tiles", "max_rows", "n_pairs", "kernel", "tile_rows")
 
 
-def moe_plan(choice: torch.Tensor, experts: int) -> ExpertRows:
+def moe_plan(choice: torch.Tensor, experts: int, kernel: str = "plain") -> ExpertRows:
     _gpu(choice)
     _need(choice.dtype == torch.int32, "choices are int32")
+    _need(kernel in MOE_KERNELS, f"kernel {kernel!r}: one of {sorted(MOE_KERNELS)}")
     lib = _load("moe")
     plan = ExpertRows()
+    plan.kernel = kernel
+    plan.tile_rows = int(lib.cw_moe_tile_rows(MOE_KERNELS[kernel]))
     plan.n_pairs = choice.numel()
-    plan.max_tiles = int(lib.cw_moe_max_tiles(plan.n_pairs, experts))
-    plan.max_rows = plan.max_tiles * int(lib.cw_moe_tile_rows())
+    plan.max_tiles = int(lib.cw_moe_max_tiles(plan.n_pairs, experts, plan.tile_rows))
+    plan.max_rows = plan.max_tiles * plan.tile_rows
     plan.row_pair = torch.empty(max(plan.max_rows, 1), dtype=torch.int32, device=choice.device)
     plan.tile_expert = torch.empty(max(plan.max_tiles, 1), dtype=torch.int32, device=choice.device)
     plan.n_tiles = torch.empty(1, dtype=torch.int32, device=choice.device)
-    _check(lib.cw_moe_plan(_ptr(choice), plan.n_pairs, experts, _ptr(plan.row_pair), plan.max_rows, _ptr(plan.tile_expert),
-                           plan.max_tiles, _ptr(plan.n_tiles), _stream()), "moe_plan")
+    _check(lib.cw_moe_plan(_ptr(choice), plan.n_pairs, experts, plan.tile_rows, _ptr(plan.row_pair), plan.max_rows,
+                           _ptr(plan.tile_expert), plan.max_tiles, _ptr(plan.n_tiles), _stream()), "moe_plan")
     return plan
 
 
@@ -1996,7 +2016,7 @@ def moe_gate_up(x: torch.Tensor, gate_up: torch.Tensor, plan: ExpertRows, score:
     _need(plan.n_pairs == T * top and score.numel() == T * top and score.dtype == torch.float32, "one score a pair")
     ff = gate_up.shape[1] // 2
     inner = torch.empty((max(plan.max_rows, 1), ff), dtype=x.dtype, device=x.device)
-    _check(_load("moe").cw_moe_expert_product(0, _ptr(x), _ptr(gate_up), _ptr(inner), dtype_code(x.dtype), _ptr(plan.row_pair),
+    _check(_load("moe").cw_moe_expert_product(0, MOE_KERNELS[plan.kernel], _ptr(x), _ptr(gate_up), _ptr(inner), dtype_code(x.dtype), _ptr(plan.row_pair),
                                               _ptr(plan.tile_expert), _ptr(plan.n_tiles), plan.max_tiles, _ptr(score), top, H, ff,
                                               int(bool(scale_input)), _stream()), "moe_gate_up")
     return inner
@@ -2011,7 +2031,7 @@ def moe_down(inner: torch.Tensor, down: torch.Tensor, plan: ExpertRows, score: t
     _need(down.dim() == 3 and down.shape[2] == ff and down.dtype == inner.dtype, "down must be [experts, H, ff] in the rows' type")
     H = down.shape[1]
     _need(inner.shape[0] >= plan.max_rows and tuple(out.shape) == (plan.n_pairs, H) and out.dtype == inner.dtype, "out must be [pairs, H]")
-    _check(_load("moe").cw_moe_expert_product(1, _ptr(inner), _ptr(down), _ptr(out), dtype_code(inner.dtype), _ptr(plan.row_pair),
+    _check(_load("moe").cw_moe_expert_product(1, MOE_KERNELS[plan.kernel], _ptr(inner), _ptr(down), _ptr(out), dtype_code(inner.dtype), _ptr(plan.row_pair),
                                               _ptr(plan.tile_expert), _ptr(plan.n_tiles), plan.max_tiles, _ptr(score), top, ff, H,
                                               int(bool(scale_output)), _stream()), "moe_down")
     return out

@@ -4,7 +4,9 @@ feed-forwards (``RoutedExpertsSpec``).
 Steps, all on the device, so a step replays as a captured graph: the router's product in float32
 with the choice of the top_k experts (one kernel); the (token, choice) pairs sorted by expert
 into rows, every expert's rows in tiles of their own (one kernel); the experts' gate and up
-products with the activation over those tiles; their down products, scattered back to the pairs;
+products with the activation over those tiles; their down products, scattered back to the pairs
+(bfloat16 on the matrix cores: tiles of 16 rows that stream an expert's matrix for steps of few
+tokens, tiles of 128 rows through LDS for portions; float32 in plain arithmetic);
 the sum over a token's pairs in float32 (not needed when top_k is 1). The experts' matrices are
 stacked: gate_up [experts, 2 * ff, hidden] (an expert's gate rows, then its up rows) and down
 [experts, hidden, ff]. Cache manager and scheduler are not involved.
@@ -42,6 +44,7 @@ class RoutedExperts(Part):
         self.router = params["router_weight"]
         self.gate_up = params["gate_up_weight"].view(s.num_experts, 2 * s.intermediate_size, s.hidden_size)
         self.down = params["down_weight"].view(s.num_experts, s.hidden_size, s.intermediate_size)
+        self.kernel = None   # a kernel's name: that one for every step (tests); None: chosen by the step's shape
 
     def route(self, x: torch.Tensor):
         """(choice int32 [T, top_k], score float32 [T, top_k])."""
@@ -52,7 +55,8 @@ class RoutedExperts(Part):
         s = self.spec
         T = x.shape[0]
         choice, score = self.route(x)
-        plan = ops.moe_plan(choice, s.num_experts)
+        kernel = self.kernel or ops.moe_kernel_for(x.dtype, T * s.top_k, s.num_experts, s.hidden_size, s.intermediate_size)
+        plan = ops.moe_plan(choice, s.num_experts, kernel)
         inner = ops.moe_gate_up(x, self.gate_up, plan, score, s.top_k, scale_input=s.weight_on == "input")
         out = torch.empty((T, s.hidden_size), dtype=x.dtype, device=x.device)
         if s.top_k == 1:

@@ -112,7 +112,8 @@ def _expert_names(w, spec):
 # hidden, ff, experts, top, tokens: one expert, all experts, more experts than tokens, more tokens of
 # an expert than a tile of rows holds, sizes that are no multiple of the kernels' tiles
 ROUTED_SHAPES = [(96, 40, 5, 2, 61), (100, 50, 2, 1, 37), (64, 1, 1, 1, 9), (48, 24, 3, 3, 130), (128, 72, 16, 4, 3),
-                 (256, 96, 8, 1, 200), (64, 130, 7, 2, 1), (72, 33, 40, 6, 20)]
+                 (256, 96, 8, 1, 200), (64, 130, 7, 2, 1), (72, 33, 40, 6, 20), (128, 64, 4, 2, 700), (72, 40, 6, 2, 33),
+                 (200, 136, 3, 1, 400)]
 
 
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
@@ -146,6 +147,36 @@ def test_routed_experts_against_the_plain_sum(dtype, shape):
         for e in mine:
             want[t] += plain.expert(r[t, e] * x[t].double(), names, f"e{e}.")
     close(part.forward(x.to(DEV), SimpleNamespace()).double().cpu(), want, dtype)
+
+
+@pytest.mark.parametrize("shape", [(72, 40, 6, 2, 33), (128, 64, 4, 2, 700), (200, 136, 3, 1, 400), (256, 96, 8, 3, 5), (64, 8, 2, 2, 130)])
+def test_the_three_kernels_of_the_experts_products_agree(shape):
+    """bfloat16: plain arithmetic, the streaming kernel and the wide tiles of the matrix cores on the
+    same step, each forced; they round alike and differ by the order of their float32 sums. Which
+    one a step takes by itself follows from its shape alone."""
+    hidden, ff, experts, top, T = shape
+    spec = RoutedExpertsSpec(hidden_size=hidden, intermediate_size=ff, num_experts=experts, top_k=top)
+    part = build_part(spec)
+    w = bind(part, torch.bfloat16, seed=experts, matrix_std=1.5 / hidden ** 0.5)
+    x = torch.randn(T, hidden, generator=torch.Generator().manual_seed(15)).to(torch.bfloat16).to(DEV)
+    names = _expert_names(w, spec)
+    choice, score = part.route(x)
+    want = torch.zeros(T, hidden, dtype=torch.float64)
+    for t in range(T):
+        for e, r in zip(choice[t].tolist(), score[t].tolist()):
+            want[t] += plain.expert(r * x[t].double().cpu(), names, f"e{e}.")
+    got = {}
+    for kernel in ("plain", "stream", "wide"):
+        part.kernel = kernel
+        got[kernel] = part.forward(x, SimpleNamespace()).double().cpu()
+        close(got[kernel], want, torch.bfloat16)
+    scale = float(want.square().mean().sqrt())
+    for kernel in ("stream", "wide"):
+        assert float((got[kernel] - got["plain"]).abs().max()) < 2e-2 * scale
+    assert ops.moe_kernel_for(torch.bfloat16, 16, 8, 1536, 4480) == "stream"
+    assert ops.moe_kernel_for(torch.bfloat16, 4096, 8, 1536, 4480) == "wide"
+    assert ops.moe_kernel_for(torch.float32, 4096, 8, 1536, 4480) == "plain"
+    assert ops.moe_kernel_for(torch.bfloat16, 4096, 8, 100, 4480) == "plain"
 
 
 def test_routing_options_and_equal_scores():
