@@ -304,6 +304,12 @@ struct WideArgs {
   int M, N, K;
   int tiles_m, tiles_n;
   int k_splits;  // MODE 3: K is cut into this many runs, each a tile of its own with a float32 plane of partial sums
+  // GROUPED: every row tile of x multiplies a matrix of its own (rows sorted by expert)
+  const int* tile_group;    // [row tiles] which of the stacked matrices a row tile takes
+  const int* n_row_tiles;   // [1] how many row tiles there are in this launch (on the device)
+  const int* row_target;    // nullptr: row m of the result is row m of C; else its row there, < 0: not stored
+  const float* row_factor;  // nullptr, or a factor for the results that go to row row_target[m]: row_factor[row_target[m]]
+  int64_t w_group_stride;   // elements from one stacked matrix to the next
 };
 
 // Row of W that row ``rb`` of W tile ``tn`` is. MODE 2: a wave's 96 rows are 48 gate rows followed
@@ -339,14 +345,16 @@ __device__ __forceinline__ uint32_t w_pack_bf16(float lo, float hi) {
     asm volatile("" ::: "memory"); \
   } while (0)
 
-template <int MODE>
+template <int MODE, bool GROUPED = false>
 __global__ __launch_bounds__(256) void gemm_wide_bf16_kernel(WideArgs a) {
   extern __shared__ __align__(1024) unsigned char w_smem[];
   const int tid = threadIdx.x, lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6);
   const int wm = wave >> 1, wn = wave & 1;
   const int c = lane & 15, s = lane >> 4;
-  const int M = a.M, N = a.N, K = a.K;
-  const int per_split = a.tiles_m * a.tiles_n;
+  // GROUPED: the number of row tiles is known on the device alone; x holds whole tiles
+  const int tiles_m = GROUPED ? __builtin_amdgcn_readfirstlane(*a.n_row_tiles) : a.tiles_m;
+  const int M = GROUPED ? tiles_m * W_BM : a.M, N = a.N, K = a.K;
+  const int per_split = tiles_m * a.tiles_n;
   const int total = per_split * (MODE == 3 ? a.k_splits : 1);
   const int xcd = blockIdx.x & 7, local = blockIdx.x >> 3, per_xcd = gridDim.x >> 3;
   const int run = total >> 3, rest = total & 7;
@@ -357,7 +365,7 @@ __global__ __launch_bounds__(256) void gemm_wide_bf16_kernel(WideArgs a) {
     if (MODE == 3) id %= per_split;  // the runs of K one after the other, each over all tiles
     const int per_group = W_GROUP_M * a.tiles_n;
     const int group = id / per_group, within = id - group * per_group;
-    const int rows = min(W_GROUP_M, a.tiles_m - group * W_GROUP_M);
+    const int rows = min(W_GROUP_M, tiles_m - group * W_GROUP_M);
     *tn = within / rows;
     *tm = group * W_GROUP_M + (within - *tn * rows);
   };
@@ -384,7 +392,8 @@ __global__ __launch_bounds__(256) void gemm_wide_bf16_kernel(WideArgs a) {
     // run's last element of the matrix's last row: rows past the end read as zeros
     xr = __builtin_amdgcn_make_buffer_rsrc((void*)(a.X + x_row0 * a.ldx + k0), 0,
                                            (int)(uint32_t)(((M - x_row0 - 1) * a.ldx + k_run) * 2), 0x00020000);
-    wr = __builtin_amdgcn_make_buffer_rsrc((void*)(a.W + w_row0 * K + k0), 0,
+    const bf16_t* w_base = GROUPED ? a.W + (int64_t)__builtin_amdgcn_readfirstlane(a.tile_group[tm]) * a.w_group_stride : a.W;
+    wr = __builtin_amdgcn_make_buffer_rsrc((void*)(w_base + w_row0 * K + k0), 0,
                                            (int)(uint32_t)(((N - w_row0 - 1) * (int64_t)K + k_run) * 2), 0x00020000);
   };
   // load i of a wave's W_LOADS for stage kt: its four x blocks, then its three W blocks
@@ -494,6 +503,7 @@ __global__ __launch_bounds__(256) void gemm_wide_bf16_kernel(WideArgs a) {
     const int out_cols = MODE == 2 ? I : N;
     constexpr int OUT_BLOCKS = MODE == 2 ? W_NB / 2 : W_NB;
     const int64_t col0 = MODE == 2 ? (int64_t)tn * (W_BN / 2) + wn * (W_BN / 4) : (int64_t)tn * W_BN + wn * (W_BN / 2);
+    float row_factor = 1.0f;  // GROUPED: of the row that is being stored
     auto packed = [&](int mi, int ni, uint32_t* lo, uint32_t* hi) __attribute__((always_inline)) {
       float v[4];
 #pragma unroll
@@ -506,6 +516,7 @@ __global__ __launch_bounds__(256) void gemm_wide_bf16_kernel(WideArgs a) {
           const int64_t n = col0 + ni * 16 + 4 * s + e;
           if (a.bias != nullptr && n < N)
             v[e] += a.bias_f32 ? ((const float*)a.bias)[n] : __bfloat162float(((const bf16_t*)a.bias)[n]);
+          if (GROUPED) v[e] *= row_factor;
         }
       }
       *lo = w_pack_bf16(v[0], v[1]);
@@ -538,7 +549,16 @@ __global__ __launch_bounds__(256) void gemm_wide_bf16_kernel(WideArgs a) {
     const bool wide_ok = !(a.ldc & 7) && !((uintptr_t)a.C & 15);
 #pragma unroll
     for (int mi = 0; mi < 8; ++mi) {
-      const int64_t m = (int64_t)tm * W_BM + wm * 128 + mi * 16 + c;
+      int64_t m = (int64_t)tm * W_BM + wm * 128 + mi * 16 + c;
+      bool live = m < M;
+      if (GROUPED && a.row_target != nullptr) {
+        // the permutes below exchange values between the lanes of one row, so a lane whose row is
+        // not stored still takes part in them
+        const int target = live ? a.row_target[m] : -1;
+        live = target >= 0;
+        row_factor = (live && a.row_factor != nullptr) ? a.row_factor[target] : 1.0f;
+        m = live ? target : 0;
+      }
 #pragma unroll
       for (int ni = 0; ni + 1 < OUT_BLOCKS; ni += 2) {
         uint32_t a_lo, a_hi, b_lo, b_hi;
@@ -549,7 +569,7 @@ __global__ __launch_bounds__(256) void gemm_wide_bf16_kernel(WideArgs a) {
         const cw_u32x2_t lo = __builtin_amdgcn_permlane16_swap(a_lo, b_lo, false, false);
         const cw_u32x2_t hi = __builtin_amdgcn_permlane16_swap(a_hi, b_hi, false, false);
         const int64_t n0 = col0 + (ni + (s & 1)) * 16 + 8 * (s >> 1);
-        if (m >= M || n0 >= out_cols) continue;
+        if (!live || n0 >= out_cols) continue;
         uint16_t* dst = (uint16_t*)a.C + m * a.ldc + n0;
         const uint32_t w4[4] = {lo[0], hi[0], lo[1], hi[1]};
         if (n0 + 8 <= out_cols && wide_ok) {
@@ -565,7 +585,7 @@ __global__ __launch_bounds__(256) void gemm_wide_bf16_kernel(WideArgs a) {
         uint32_t lo, hi;
         packed(mi, ni, &lo, &hi);
         const int64_t n0 = col0 + ni * 16 + 4 * s;
-        if (m >= M || n0 >= out_cols) continue;
+        if (!live || n0 >= out_cols) continue;
         uint16_t* dst = (uint16_t*)a.C + m * a.ldc + n0;
         if (n0 + 4 <= out_cols && !(a.ldc & 3)) {
           *reinterpret_cast<uint2*>(dst) = make_uint2(lo, hi);
@@ -650,3 +670,50 @@ CW_EXPORT int cw_gemm_bf16_wide_partial(const void* X, int64_t ldx, const void* 
   WideArgs a{(const bf16_t*)X, ldx, (const bf16_t*)W, nullptr, 0, parts, ldc, M, N, K, 0, 0, k_splits};
   return w_launch<3>(a, workgroups, stream);
 }
+
+template <int MODE>
+static int w_launch_grouped(WideArgs a, int max_row_tiles, int workgroups, hipStream_t stream) {
+  static bool raised = false;
+  if (!raised) {
+    if (hipFuncSetAttribute((const void*)gemm_wide_bf16_kernel<MODE, true>, hipFuncAttributeMaxDynamicSharedMemorySize,
+                            (int)W_SMEM) != hipSuccess)
+      return CW_ERR_LAUNCH;
+    raised = true;
+  }
+  const int out_cols = MODE == 2 ? a.N / 2 : a.N;
+  const int per_tile = MODE == 2 ? W_BN / 2 : W_BN;
+  a.tiles_n = (out_cols + per_tile - 1) / per_tile;
+  a.tiles_m = 0;  // read on the device
+  const int64_t most = (int64_t)max_row_tiles * a.tiles_n;
+  int grid = most < workgroups ? (int)most : workgroups;
+  grid = (grid + 7) & ~7;
+  hipLaunchKernelGGL((gemm_wide_bf16_kernel<MODE, true>), dim3(grid), dim3(256), W_SMEM, stream, a);
+  return cw_launch_status();
+}
+
+// Products of row tiles with matrices of their own through the wide-tile kernel: x holds
+// ``*n_row_tiles`` (at most ``max_row_tiles``, a number on the device) tiles of 256 rows, and tile t
+// multiplies matrix ``tile_group[t]`` of the stack W [groups, N, K] (``w_group_stride`` elements
+// apart). mode 0: C[row_target[m]] = x[m] W_g^T (times row_factor[row_target[m]] when given; rows
+// whose target is negative are not stored; row_target nullptr: C[m]). mode 2: W_g = [gate; up],
+// C[m, i] = silu(gate_i . x_m) * (up_i . x_m). The grid depends on max_row_tiles alone, so a
+// captured launch replays with other numbers of tiles. K a multiple of 64, at least 256.
+CW_EXPORT int cw_gemm_bf16_wide_grouped(int mode, const void* X, int64_t ldx, const void* W, int64_t w_group_stride,
+                                        void* C, int64_t ldc, int N, int K, const int* tile_group, const int* n_row_tiles,
+                                        int max_row_tiles, const int* row_target, const float* row_factor, int workgroups,
+                                        hipStream_t stream) {
+  if (N <= 0 || K <= 0 || (mode != 0 && mode != 2) || workgroups < 8 || max_row_tiles < 0) return CW_ERR_ARG;
+  if (!X || !W || !C || !tile_group || !n_row_tiles || (row_factor && !row_target)) return CW_ERR_ARG;
+  if (((uintptr_t)X & 15) || ((uintptr_t)W & 15) || ((uintptr_t)C & 7) || (w_group_stride & 7)) return CW_ERR_ARG;
+  if (mode == 2 && (N & 1)) return CW_ERR_ARG;
+  if (ldc < (mode == 2 ? N / 2 : N) || w_group_stride < (int64_t)N * K) return CW_ERR_ARG;
+  if (max_row_tiles == 0) return CW_OK;
+  if (cw_gemm_bf16_wide_tiles(mode, max_row_tiles * W_BM, N, K, ldx) == 0) return CW_ERR_SIZE;
+  WideArgs a{(const bf16_t*)X, ldx, (const bf16_t*)W, nullptr, 0, C, ldc, 0, N, K, 0, 0, 1,
+             tile_group, n_row_tiles, row_target, row_factor, w_group_stride};
+  return mode == 2 ? w_launch_grouped<2>(a, max_row_tiles, workgroups, stream)
+                   : w_launch_grouped<0>(a, max_row_tiles, workgroups, stream);
+}
+
+// rows of a tile of cw_gemm_bf16_wide_grouped
+CW_EXPORT int cw_gemm_bf16_wide_rows(void) { return W_BM; }

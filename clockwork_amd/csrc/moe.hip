@@ -31,6 +31,7 @@ typedef __attribute__((ext_vector_type(4))) unsigned int u32x4_t;
 
 #define MOE_TILE_ROWS 16    // of the plain and the streaming kernel
 #define MOE_WIDE_ROWS 128   // of the LDS-tiled kernel
+#define MOE_GROUPED_ROWS 256  // of the matrix product over row tiles with matrices of their own (another library's)
 #define MOE_MAX_EXPERTS 1024
 #define MOE_ROUTER_SIGMOID 0
 #define MOE_ROUTER_SOFTMAX 1
@@ -44,10 +45,31 @@ __global__ __launch_bounds__(256) void moe_route_kernel(const T* __restrict__ x,
   const int64_t t = blockIdx.x;
   const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
   const T* xr = x + t * H;
+  constexpr int V = 16 / (int)sizeof(T);
+  const bool vec_ok = H % V == 0 && !((uintptr_t)x & 15) && !((uintptr_t)router & 15);
   for (int e = wave; e < E; e += 4) {
     const T* w = router + (int64_t)e * H;
     float s = 0.0f;
-    for (int j = lane; j < H; j += 64) s += cw_to_float(xr[j]) * cw_to_float(w[j]);
+    if (vec_ok) {  // 16 bytes of each row a lane and step; the order of a lane's sums depends on H alone
+      for (int j = lane * V; j < H; j += 64 * V) {
+        if constexpr (sizeof(T) == 4) {
+          const f32x4_t a = *reinterpret_cast<const f32x4_t*>(xr + j);
+          const f32x4_t b = *reinterpret_cast<const f32x4_t*>(w + j);
+#pragma unroll
+          for (int i = 0; i < 4; ++i) s += a[i] * b[i];
+        } else {
+          const u32x4_t a = *reinterpret_cast<const u32x4_t*>(xr + j);
+          const u32x4_t b = *reinterpret_cast<const u32x4_t*>(w + j);
+#pragma unroll
+          for (int i = 0; i < 4; ++i) {
+            s += cw_bf16_bits_to_float((uint16_t)(a[i] & 0xffffu)) * cw_bf16_bits_to_float((uint16_t)(b[i] & 0xffffu));
+            s += cw_bf16_bits_to_float((uint16_t)(a[i] >> 16)) * cw_bf16_bits_to_float((uint16_t)(b[i] >> 16));
+          }
+        }
+      }
+    } else {
+      for (int j = lane; j < H; j += 64) s += cw_to_float(xr[j]) * cw_to_float(w[j]);
+    }
     s = cw_wave_sum(s);
     if (lane == 0) r[e] = s;
   }
@@ -492,6 +514,40 @@ __global__ __launch_bounds__(256, 2) void moe_wide_bf16_kernel(const bf16_t* __r
   }
 }
 
+// ---------------------------------------------------------------- 3a. the rows of the experts' tiles, laid out
+// rows[r] = x[token of pair row_pair[r]] (times the pair's score with ``use_score``, rounded to
+// bfloat16 as the other kernels round it), zeros where a row holds no pair; only the rows of the
+// tiles that exist are written. For a matrix product that reads its rows as they lie (the grouped
+// product of gemm_tile.hip). A workgroup takes rows in turn; 8 elements a thread.
+__global__ __launch_bounds__(256) void moe_gather_bf16_kernel(const bf16_t* __restrict__ x, bf16_t* __restrict__ rows,
+                                                              const int* __restrict__ row_pair,
+                                                              const int* __restrict__ n_tiles, int tile_rows,
+                                                              const float* __restrict__ score, int top, int K,
+                                                              int use_score) {
+  const int n_rows = *n_tiles * tile_rows;
+  for (int r = blockIdx.x; r < n_rows; r += gridDim.x) {
+    const int p = row_pair[r];
+    const float f = (p >= 0 && use_score) ? score[p] : 1.0f;
+    const bf16_t* src = x + (int64_t)(p >= 0 ? p / top : 0) * K;
+    bf16_t* dst = rows + (int64_t)r * K;
+    for (int k = threadIdx.x * 8; k < K; k += 256 * 8) {
+      u32x4_t v = (u32x4_t){0u, 0u, 0u, 0u};
+      if (p >= 0) {
+        v = *reinterpret_cast<const u32x4_t*>(src + k);
+        if (use_score) {
+#pragma unroll
+          for (int j = 0; j < 4; ++j) {
+            const float lo = cw_bf16_bits_to_float((uint16_t)(v[j] & 0xffffu)) * f;
+            const float hi = cw_bf16_bits_to_float((uint16_t)(v[j] >> 16)) * f;
+            v[j] = (uint32_t)cw_float_to_bf16_bits(lo) | ((uint32_t)cw_float_to_bf16_bits(hi) << 16);
+          }
+        }
+      }
+      *reinterpret_cast<u32x4_t*>(dst + k) = v;
+    }
+  }
+}
+
 // ---------------------------------------------------------------- 5. a token's pairs, added in their order
 template <typename T>
 __global__ void moe_combine_kernel(const T* __restrict__ y, T* __restrict__ out, int top, int H, int64_t total) {
@@ -506,7 +562,9 @@ __global__ void moe_combine_kernel(const T* __restrict__ y, T* __restrict__ out,
 
 // ---------------------------------------------------------------- entry points
 // rows of a tile by kernel: 0 plain arithmetic, 1 streaming (matrix cores), 2 wide tiles (matrix cores)
-CW_EXPORT int cw_moe_tile_rows(int kernel) { return kernel == 2 ? MOE_WIDE_ROWS : MOE_TILE_ROWS; }
+CW_EXPORT int cw_moe_tile_rows(int kernel) {
+  return kernel == 3 ? MOE_GROUPED_ROWS : kernel == 2 ? MOE_WIDE_ROWS : MOE_TILE_ROWS;
+}
 
 // the most tiles that ``n_pairs`` pairs over ``E`` experts can need
 CW_EXPORT int cw_moe_max_tiles(int n_pairs, int E, int tile_rows) {
@@ -534,7 +592,7 @@ CW_EXPORT int cw_moe_route(const void* x, const void* router, int dtype, int T, 
 CW_EXPORT int cw_moe_plan(const int* choice, int n_pairs, int E, int tile_rows, int* row_pair, int max_rows, int* tile_expert,
                           int max_tiles, int* n_tiles, hipStream_t stream) {
   if (n_pairs < 0 || E <= 0 || !choice || !row_pair || !tile_expert || !n_tiles) return CW_ERR_ARG;
-  if (tile_rows != MOE_TILE_ROWS && tile_rows != MOE_WIDE_ROWS) return CW_ERR_ARG;
+  if (tile_rows != MOE_TILE_ROWS && tile_rows != MOE_WIDE_ROWS && tile_rows != MOE_GROUPED_ROWS) return CW_ERR_ARG;
   if (E > MOE_MAX_EXPERTS) return CW_ERR_SIZE;
   if (max_tiles < cw_moe_max_tiles(n_pairs, E, tile_rows) || max_rows < max_tiles * tile_rows) return CW_ERR_ARG;
   hipLaunchKernelGGL(moe_plan_kernel, dim3(1), dim3(1024), 0, stream, choice, n_pairs, E, tile_rows, max_rows, row_pair,
@@ -596,6 +654,22 @@ CW_EXPORT int cw_moe_expert_product(int mode, int kernel, const void* x, const v
   else if (dtype == CW_BF16 && mode == 1) CW_LAUNCH(bf16_t, 1);
   else return CW_ERR_DTYPE;
 #undef CW_LAUNCH
+  return cw_launch_status();
+}
+
+// rows [max_tiles * tile_rows, K] bfloat16 = the plan's rows of x [tokens, K] as they lie, for a
+// product that gathers nothing (K a multiple of 8)
+CW_EXPORT int cw_moe_gather(const void* x, void* rows, int dtype, const int* row_pair, const int* n_tiles, int max_tiles,
+                            int tile_rows, const float* score, int top, int K, int use_score, hipStream_t stream) {
+  if (max_tiles < 0 || tile_rows <= 0 || K <= 0 || top <= 0 || !x || !rows || !row_pair || !n_tiles) return CW_ERR_ARG;
+  if (use_score && !score) return CW_ERR_ARG;
+  if (dtype != CW_BF16) return CW_ERR_DTYPE;
+  if ((K & 7) || ((uintptr_t)x & 15) || ((uintptr_t)rows & 15)) return CW_ERR_ARG;
+  if (max_tiles == 0) return CW_OK;
+  int64_t blocks = (int64_t)max_tiles * tile_rows;
+  if (blocks > 4096) blocks = 4096;
+  hipLaunchKernelGGL(moe_gather_bf16_kernel, dim3((unsigned)blocks), dim3(256), 0, stream, (const bf16_t*)x, (bf16_t*)rows,
+                     row_pair, n_tiles, tile_rows, score, top, K, use_score);
   return cw_launch_status();
 }
 

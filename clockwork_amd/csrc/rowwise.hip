@@ -750,12 +750,12 @@ CW_EXPORT int cw_stream_norm(const float* resid, const void* w, int w_dtype, flo
 // cache row. One workgroup a token, one wave a vector at a time; float32 inside.
 #define HN_MAX_DIM 1024
 template <typename T, typename WT, typename BT>
-__global__ __launch_bounds__(256) void headnorm_rope_store_kernel(
+__global__ __launch_bounds__(1024) void headnorm_rope_store_kernel(
     T* __restrict__ proj, int64_t stride, int q_off, int k_off, int v_off, int nqv, int nkv, int dim, int nv,
     const BT* __restrict__ bias, const WT* __restrict__ qw, const WT* __restrict__ kw, float eps,
     const int* __restrict__ positions, const float* __restrict__ freq, int rdims, const int* __restrict__ slots,
     T* __restrict__ k_plane, T* __restrict__ v_plane, int v_from_keys, int64_t cache_rows) {
-  extern __shared__ float hn_vals[];  // [4 waves][dim]
+  extern __shared__ float hn_vals[];  // [waves][dim], then the token's cosines and sines [2][rdims / 2]
   const int64_t t = blockIdx.x;
   T* row = proj + t * stride;
   int64_t slot = slots ? (int64_t)slots[t] : -1;
@@ -764,13 +764,18 @@ __global__ __launch_bounds__(256) void headnorm_rope_store_kernel(
   if (slot >= 0 && v_plane) {
     const int src = v_from_keys ? k_off : v_off;
     T* vd = v_plane + slot * nv;
-    for (int j = threadIdx.x; j < nv; j += 256)
+    for (int j = threadIdx.x; j < nv; j += blockDim.x)
       vd[j] = cw_from_float<T>(cw_to_float(row[src + j]) + (bias ? cw_to_float(bias[src + j]) : 0.0f));
   }
   const float pos = positions ? (float)positions[t] : 0.0f;
-  const int half = rdims / 2;
+  const int half = rdims / 2, n_waves = blockDim.x >> 6;
   float* vals = hn_vals + wave * dim;
-  for (int vec = wave; vec < nqv + nkv; vec += 4) {
+  // the angles are the same for every vector of the token: made once
+  float* cosines = hn_vals + n_waves * dim;
+  float* sines = cosines + half;
+  for (int i = threadIdx.x; i < half; i += blockDim.x) sincosf(pos * freq[i], &sines[i], &cosines[i]);
+  __syncthreads();
+  for (int vec = wave; vec < nqv + nkv; vec += n_waves) {
     const bool is_q = vec < nqv;
     if (!is_q && slot < 0) continue;
     const int base = is_q ? q_off + vec * dim : k_off + (vec - nqv) * dim;
@@ -792,8 +797,7 @@ __global__ __launch_bounds__(256) void headnorm_rope_store_kernel(
         const int i = j < half ? j : j - half;
         const float a = vals[i] * inv * (w ? cw_to_float(w[i]) : 1.0f);
         const float b = vals[i + half] * inv * (w ? cw_to_float(w[i + half]) : 1.0f);
-        float s, c;
-        sincosf(pos * freq[i], &s, &c);
+        const float s = sines[i], c = cosines[i];
         v = j < half ? a * c - b * s : b * c + a * s;
       } else {
         v = vals[j] * inv * (w ? cw_to_float(w[j]) : 1.0f);
@@ -819,8 +823,12 @@ CW_EXPORT int cw_headnorm_rope_store(void* proj, int dtype, int64_t stride, int 
   if (!proj || (rdims && (!freq || !positions)) || (slots && nkv && !k_plane) || (slots && nv && !v_plane)) return CW_ERR_ARG;
   if ((qw == nullptr) != (kw == nullptr)) return CW_ERR_ARG;
   if (T == 0) return CW_OK;
-  dim3 grid(T), block(256);
-  const size_t lds = (size_t)4 * dim * sizeof(float);
+  // a wave a vector at a time: as many waves as there are vectors, 4 to 16
+  const int n_vec = nqv + nkv;
+  int waves = n_vec < 4 ? 4 : n_vec > 16 ? 16 : n_vec;
+  while (waves > 4 && ((size_t)waves * dim + rdims) * sizeof(float) > 49152) --waves;  // their vectors share 48 KB of LDS
+  dim3 grid(T), block(64 * waves);
+  const size_t lds = ((size_t)waves * dim + rdims) * sizeof(float);
 #define CW_LAUNCH(T_, WT_, BT_)                                                                                          \
   hipLaunchKernelGGL((headnorm_rope_store_kernel<T_, WT_, BT_>), grid, block, lds, stream, (T_*)proj, stride, q_off, k_off, \
                      v_off, nqv, nkv, dim, nv, (const BT_*)bias, (const WT_*)qw, (const WT_*)kw, eps, positions, freq, rdims, \

@@ -117,6 +117,7 @@ def _declare(name: str, lib: ctypes.CDLL) -> None:
             "cw_gemm_bf16_wide": [I, P, L, P, P, I, P, L, I, I, I, I, P],
             "cw_gemm_bf16_wide_partial_ok": [I, I, I, L, I],
             "cw_gemm_bf16_wide_partial": [P, L, P, P, L, I, I, I, I, I, P],
+            "cw_gemm_bf16_wide_grouped": [I, P, L, P, L, P, L, I, I, P, P, I, P, P, I, P],
         },
         "rowwise": {
             "cw_embedding_pos": [P, I, P, P, P, F, P, I, I, I, I, P],
@@ -144,6 +145,7 @@ def _declare(name: str, lib: ctypes.CDLL) -> None:
             "cw_moe_route": [P, P, I, I, I, I, I, I, I, P, P, P],
             "cw_moe_plan": [P, I, I, I, P, I, P, I, P, P],
             "cw_moe_expert_product": [I, I, P, P, P, I, P, P, P, I, P, I, I, I, I, P],
+            "cw_moe_gather": [P, P, I, P, P, I, I, P, I, I, I, P],
             "cw_moe_combine": [P, P, I, I, I, I, P],
         },
         "rows_attention": {
@@ -1960,9 +1962,11 @@ def moe_route(x: torch.Tensor, router: torch.Tensor, top: int, kind: str = "sigm
     return choice, score
 
 
-MOE_KERNELS = {"plain": 0, "stream": 1, "wide": 2}
+MOE_KERNELS = {"plain": 0, "stream": 1, "wide": 2, "grouped": 3}
 # rows an expert from which a step's experts run on the wide tiles of the matrix-core kernel
 MOE_WIDE_FROM = 48
+# rows an expert from which they run as row tiles of the dense products' wide-tile kernel
+MOE_GROUPED_FROM = 256
 
 
 def moe_kernel_for(dtype, n_pairs: int, experts: int, hidden: int, ff: int) -> str:
@@ -1970,10 +1974,21 @@ def moe_kernel_for(dtype, n_pairs: int, experts: int, hidden: int, ff: int) -> s
     (never by what the router chose), so a captured step replays. bfloat16 with widths that are a
     multiple of 8 runs on the matrix cores: "wide" tiles of 128 rows from ``MOE_WIDE_FROM`` rows an
     expert on average, else "stream" (tiles of 16 rows, the expert's matrix read once a tile);
-    everything else, float32 included, "plain" arithmetic."""
+    from ``MOE_GROUPED_FROM`` rows an expert, with widths that are a multiple of 64 and at least 256,
+    "grouped": the rows laid out expert by expert in tiles of 256 and multiplied by the kernel of
+    the dense products of long portions, every row tile with its expert's matrix. Everything else,
+    float32 included, "plain" arithmetic."""
     if dtype != torch.bfloat16 or hidden % 8 or ff % 8:
         return "plain"
+    grouped_rows = (n_pairs // 256 + min(n_pairs, experts)) * 256   # the most rows its tiles can hold
+    if n_pairs >= MOE_GROUPED_FROM * experts and moe_grouped_ok(hidden, ff) and grouped_rows * max(hidden, ff) * 2 < 2 ** 32:
+        return "grouped"
     return "wide" if n_pairs >= MOE_WIDE_FROM * experts else "stream"
+
+
+def moe_grouped_ok(hidden: int, ff: int) -> bool:
+    """Does the grouped product take experts of these widths (both are a K of one of its products)?"""
+    return min(hidden, ff) >= 256 and hidden % 64 == 0 and ff % 64 == 0 and 2 * ff * hidden * 2 < 2 ** 32
 
 
 class ExpertRows:
@@ -2016,6 +2031,16 @@ def moe_gate_up(x: torch.Tensor, gate_up: torch.Tensor, plan: ExpertRows, score:
     _need(plan.n_pairs == T * top and score.numel() == T * top and score.dtype == torch.float32, "one score a pair")
     ff = gate_up.shape[1] // 2
     inner = torch.empty((max(plan.max_rows, 1), ff), dtype=x.dtype, device=x.device)
+    if plan.kernel == "grouped":
+        _need(x.dtype == torch.bfloat16 and moe_grouped_ok(H, ff), "the grouped product takes bfloat16 and widths that are a multiple of 64")
+        rows = torch.empty((max(plan.max_rows, 1), H), dtype=x.dtype, device=x.device)
+        _check(_load("moe").cw_moe_gather(_ptr(x), _ptr(rows), dtype_code(x.dtype), _ptr(plan.row_pair), _ptr(plan.n_tiles),
+                                          plan.max_tiles, plan.tile_rows, _ptr(score), top, H, int(bool(scale_input)), _stream()),
+               "moe_gather")
+        _check(_load("gemm_tile").cw_gemm_bf16_wide_grouped(2, _ptr(rows), H, _ptr(gate_up), gate_up.stride(0), _ptr(inner), ff,
+                                                            2 * ff, H, _ptr(plan.tile_expert), _ptr(plan.n_tiles), plan.max_tiles,
+                                                            None, None, _compute_units(x.device), _stream()), "moe_gate_up")
+        return inner
     _check(_load("moe").cw_moe_expert_product(0, MOE_KERNELS[plan.kernel], _ptr(x), _ptr(gate_up), _ptr(inner), dtype_code(x.dtype), _ptr(plan.row_pair),
                                               _ptr(plan.tile_expert), _ptr(plan.n_tiles), plan.max_tiles, _ptr(score), top, H, ff,
                                               int(bool(scale_input)), _stream()), "moe_gate_up")
@@ -2031,6 +2056,13 @@ def moe_down(inner: torch.Tensor, down: torch.Tensor, plan: ExpertRows, score: t
     _need(down.dim() == 3 and down.shape[2] == ff and down.dtype == inner.dtype, "down must be [experts, H, ff] in the rows' type")
     H = down.shape[1]
     _need(inner.shape[0] >= plan.max_rows and tuple(out.shape) == (plan.n_pairs, H) and out.dtype == inner.dtype, "out must be [pairs, H]")
+    if plan.kernel == "grouped":
+        _need(inner.dtype == torch.bfloat16 and moe_grouped_ok(H, ff) and inner.is_contiguous(), "the grouped product takes bfloat16 and widths that are a multiple of 64")
+        _check(_load("gemm_tile").cw_gemm_bf16_wide_grouped(0, _ptr(inner), ff, _ptr(down), down.stride(0), _ptr(out), H, H, ff,
+                                                            _ptr(plan.tile_expert), _ptr(plan.n_tiles), plan.max_tiles,
+                                                            _ptr(plan.row_pair), _ptr(score) if scale_output else None,
+                                                            _compute_units(inner.device), _stream()), "moe_down")
+        return out
     _check(_load("moe").cw_moe_expert_product(1, MOE_KERNELS[plan.kernel], _ptr(inner), _ptr(down), _ptr(out), dtype_code(inner.dtype), _ptr(plan.row_pair),
                                               _ptr(plan.tile_expert), _ptr(plan.n_tiles), plan.max_tiles, _ptr(score), top, ff, H,
                                               int(bool(scale_output)), _stream()), "moe_down")

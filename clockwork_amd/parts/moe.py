@@ -37,7 +37,10 @@ class RoutedExperts(Part):
         }
 
     def kernel_libraries(self) -> list:
-        return [("moe", None)]
+        s = self.spec
+        # long portions of experts wide enough run through the dense products' wide-tile kernel
+        grouped = ops.moe_grouped_ok(s.hidden_size, s.intermediate_size)
+        return [("moe", None)] + ([("gemm_tile", None)] if grouped else [])
 
     def bind(self, params, device, dtype) -> None:
         s = self.spec

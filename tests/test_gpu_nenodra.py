@@ -174,9 +174,56 @@ def test_the_three_kernels_of_the_experts_products_agree(shape):
     for kernel in ("stream", "wide"):
         assert float((got[kernel] - got["plain"]).abs().max()) < 2e-2 * scale
     assert ops.moe_kernel_for(torch.bfloat16, 16, 8, 1536, 4480) == "stream"
-    assert ops.moe_kernel_for(torch.bfloat16, 4096, 8, 1536, 4480) == "wide"
+    assert ops.moe_kernel_for(torch.bfloat16, 1024, 8, 1536, 4480) == "wide"
+    assert ops.moe_kernel_for(torch.bfloat16, 4096, 8, 1536, 4480) == "grouped"
+    assert ops.moe_kernel_for(torch.bfloat16, 4096, 8, 1536, 4488) == "wide"
     assert ops.moe_kernel_for(torch.float32, 4096, 8, 1536, 4480) == "plain"
     assert ops.moe_kernel_for(torch.bfloat16, 4096, 8, 100, 4480) == "plain"
+
+
+@pytest.mark.parametrize("weight_on", ["input", "output"])
+@pytest.mark.parametrize("shape", [(256, 320, 3, 2, 700), (320, 256, 5, 1, 300), (448, 256, 2, 2, 1030), (256, 256, 6, 3, 90)])
+def test_the_experts_as_row_tiles_of_the_dense_products_kernel(shape, weight_on):
+    """bfloat16, widths that are multiples of 64: the rows laid out expert by expert in tiles of 256
+    and multiplied by the wide-tile kernel of the dense products, every tile with its expert's
+    matrices; experts with more than a tile of rows, with a part of one, with none (the router of
+    one expert is turned away from every token). Against the plain sum and the plain-arithmetic
+    kernel, with the score on the expert's input and on its output."""
+    hidden, ff, experts, top, T = shape
+    spec = RoutedExpertsSpec(hidden_size=hidden, intermediate_size=ff, num_experts=experts, top_k=top, weight_on=weight_on)
+    part = build_part(spec)
+
+    def change(v):
+        if experts > top + 1:
+            v["router_weight"][experts - 2] = -8.0 * v["router_weight"][experts - 2].abs()   # with inputs > 0: never chosen
+
+    w = bind(part, torch.bfloat16, seed=experts + 1, matrix_std=1.5 / hidden ** 0.5, change=change)
+    x = (torch.randn(T, hidden, generator=torch.Generator().manual_seed(16)).abs() + 0.05).to(torch.bfloat16).to(DEV)
+    names = _expert_names(w, spec)
+    choice, score = part.route(x)
+    if experts > top + 1:
+        assert not bool((choice == experts - 2).any())
+    want = torch.zeros(T, hidden, dtype=torch.float64)
+    for t in range(T):
+        for e, r in zip(choice[t].tolist(), score[t].tolist()):
+            xt = x[t].double().cpu()
+            want[t] += (r * plain.expert(xt, names, f"e{e}.") if weight_on == "output"
+                        else plain.expert((r * xt).to(torch.bfloat16).double(), names, f"e{e}."))
+    got = {}
+    for kernel in ("plain", "grouped"):
+        part.kernel = kernel
+        got[kernel] = part.forward(x, SimpleNamespace()).double().cpu()
+        close(got[kernel], want, torch.bfloat16)
+    scale = float(want.square().mean().sqrt())
+    # both round a value to bfloat16 once: they differ by the order of their float32 sums, which
+    # moves an element by one step of its last bit at most
+    assert float(((got["grouped"] - got["plain"]).abs() / (got["plain"].abs() + scale)).max()) < 2e-2
+    # a second step of other tokens through the same part: fewer rows, other experts' tiles
+    x2 = x[: max(T // 3, 1)].flip(0).contiguous()
+    part.kernel = "plain"
+    want2 = part.forward(x2, SimpleNamespace()).double().cpu()
+    part.kernel = "grouped"
+    assert float(((part.forward(x2, SimpleNamespace()).double().cpu() - want2).abs() / (want2.abs() + scale)).max()) < 2e-2
 
 
 def test_routing_options_and_equal_scores():
