@@ -198,7 +198,7 @@ CW_EXPORT int cw_gemm_f32(const float* A, int64_t lda, const float* W, const flo
 // k at slot l/16), and 16 tokens x the same k-values as the B operand.
 //
 // MODE 0: y bfloat16 [M, N]; MODE 4: the same with the erf GELU applied to the float32 sums before
-// they are rounded; MODE 1: y float32 [M, N] (logits); MODE 2: W is [2I, K] with gate
+// they are rounded; MODE 5: with max(z, 0)^2 applied to them; MODE 1: y float32 [M, N] (logits); MODE 2: W is [2I, K] with gate
 // rows first, y[m, i] = silu(gate_i) * up_i as bfloat16 [M, I]: a row tile holds 8 gate rows and
 // the 8 up rows that belong to them. MODE 3: K is also split over gridDim.y workgroups, each
 // writing its float32 partial product [split, M, N]; whoever reads y next sums the partials in
@@ -226,6 +226,7 @@ __device__ __forceinline__ bf16x8_t cw_to_operand_layout(const bf16x8_t& v, int 
 }
 
 __device__ __forceinline__ float cw_gelu_erf(float z) { return 0.5f * z * (1.0f + erff(z * 0.70710678118654752440f)); }
+__device__ __forceinline__ float cw_relu_squared(float z) { const float r = fmaxf(z, 0.0f); return r * r; }
 
 // ROWS (16, 8 or 4) is the number of weight rows a tile really holds: a narrow output with a long K
 // is cut into more, smaller tiles so that every compute unit streams a share of the matrix (the
@@ -350,6 +351,7 @@ __global__ __launch_bounds__(WAVES * 64) void gemm_skinny_bf16_kernel(const bf16
       if (MODE == 3) ((float*)C)[((int64_t)blockIdx.y * M + m) * ldc + n] = v;
       else if (MODE == 1) ((float*)C)[(int64_t)m * ldc + n] = v;
       else if (MODE == 4) ((bf16_t*)C)[(int64_t)m * ldc + n] = __float2bfloat16(cw_gelu_erf(v));
+      else if (MODE == 5) ((bf16_t*)C)[(int64_t)m * ldc + n] = __float2bfloat16(cw_relu_squared(v));
       else ((bf16_t*)C)[(int64_t)m * ldc + n] = __float2bfloat16(v);
     }
   }
@@ -517,6 +519,7 @@ __global__ __launch_bounds__(WAVES * 64) void gemm_stream_bf16_kernel(const bf16
           if (MODE == 3) ((float*)C)[((int64_t)blockIdx.y * M + m) * ldc + n] = v;
           else if (MODE == 1) ((float*)C)[(int64_t)m * ldc + n] = v;
           else if (MODE == 4) ((bf16_t*)C)[(int64_t)m * ldc + n] = __float2bfloat16(cw_gelu_erf(v));
+          else if (MODE == 5) ((bf16_t*)C)[(int64_t)m * ldc + n] = __float2bfloat16(cw_relu_squared(v));
           else ((bf16_t*)C)[(int64_t)m * ldc + n] = __float2bfloat16(v);
         }
       }
@@ -676,6 +679,7 @@ static int try_stream(int mode, const bf16_t* X, int64_t ldx, const bf16_t* W, v
     case 1: return launch_stream_mt<1, 16>(mt, spw, grid, X, ldx, W, C, ldc, M, N, K, n_tiles, stream);
     case 2: return launch_stream_mt<2, 16>(mt, spw, grid, X, ldx, W, C, ldc, M, N, K, n_tiles, stream);
     case 4: return launch_stream_mt<4, 16>(mt, spw, grid, X, ldx, W, C, ldc, M, N, K, n_tiles, stream);
+    case 5: return launch_stream_mt<5, 16>(mt, spw, grid, X, ldx, W, C, ldc, M, N, K, n_tiles, stream);
     default: return launch_stream_mt<3, 8>(mt, spw, grid, X, ldx, W, C, ldc, M, N, K, n_tiles, stream);
   }
 }
@@ -692,6 +696,7 @@ static int launch_skinny(int mode, const bf16_t* X, int64_t ldx, const bf16_t* W
   else if (mode == 1) hipLaunchKernelGGL((gemm_skinny_bf16_kernel<MT, RT, 1, WAVES, ROWS>), grid, block, 0, stream, X, ldx, W, C, ldc, M, N, K);
   else if (mode == 3) hipLaunchKernelGGL((gemm_skinny_bf16_kernel<MT, RT, 3, WAVES, ROWS>), grid, block, 0, stream, X, ldx, W, C, ldc, M, N, K);
   else if (mode == 4) hipLaunchKernelGGL((gemm_skinny_bf16_kernel<MT, RT, 4, WAVES, ROWS>), grid, block, 0, stream, X, ldx, W, C, ldc, M, N, K);
+  else if (mode == 5) hipLaunchKernelGGL((gemm_skinny_bf16_kernel<MT, RT, 5, WAVES, ROWS>), grid, block, 0, stream, X, ldx, W, C, ldc, M, N, K);
   else if (ROWS == 16) hipLaunchKernelGGL((gemm_skinny_bf16_kernel<MT, RT, 2, WAVES, 16>), grid, block, 0, stream, X, ldx, W, C, ldc, M, N, K);
   else return CW_ERR_ARG;
   return cw_launch_status();
@@ -745,7 +750,7 @@ CW_EXPORT int cw_gemm_bf16_skinny_ksplits(int M, int N, int K) {
 // that range run, but a library product is faster). mode 3 is answered by ..._ksplits() > 1.
 CW_EXPORT int cw_gemm_bf16_skinny_fast(int mode, int M, int N, int K) {
   if (M <= 16) return 1;
-  if (mode < 0 || (mode > 2 && mode != 4)) return 0;
+  if (mode < 0 || (mode > 2 && mode != 4 && mode != 5)) return 0;
   int mt, spw, n_tiles;
   dim3 grid;
   return plan_stream(mode, M, N, K, 1, &mt, &spw, &grid, &n_tiles) ? 1 : 0;
@@ -792,13 +797,13 @@ CW_EXPORT int cw_gemm_bf16_swiglu_normed(const float* resid, const void* delta, 
 }
 
 // y = x W^T for M <= 64 rows of bfloat16 x [M, K] (row stride ldx) and bfloat16 W [N, K].
-// mode 0: y bfloat16 [M, N]; 1: y float32 [M, N]; 2: y = silu(gate) * up, bfloat16 [M, N / 2];
+// mode 0: y bfloat16 [M, N] (4: gelu(y), the erf form; 5: max(y, 0)^2); 1: y float32 [M, N]; 2: y = silu(gate) * up, bfloat16 [M, N / 2];
 // 3: float32 partial products [splits, M, N], splits = ``k_splits`` if that is positive (up to 16
 // rows of x; what a caller has measured to be the best for the shape), else
 // cw_gemm_bf16_skinny_ksplits(M, N, K). K must be a multiple of 8 (16-byte rows).
 CW_EXPORT int cw_gemm_bf16_skinny(int mode, const void* X, int64_t ldx, const void* W, void* C,
                                   int64_t ldc, int M, int N, int K, int k_splits, hipStream_t stream) {
-  if (M < 0 || N <= 0 || K <= 0 || mode < 0 || mode > 4) return CW_ERR_ARG;
+  if (M < 0 || N <= 0 || K <= 0 || mode < 0 || mode > 5) return CW_ERR_ARG;
   if (M > CW_SKINNY_MAX_M) return CW_ERR_SIZE;
   if ((K & 7) || (ldx & 7) || ((uintptr_t)X & 15) || ((uintptr_t)W & 15)) return CW_ERR_ARG;
   if (mode == 2 && (N & 1)) return CW_ERR_ARG;

@@ -273,7 +273,8 @@ CW_EXPORT int cw_gemm_bf16_tiled(int mode, const void* X, int64_t ldx, const voi
 // change places between lane rows (v_permlane16_swap) so that it stores 16 bytes and four lanes
 // 64 bytes of a row.
 //
-// MODE as above; K a multiple of 64, at least 256; both matrices below 4 GiB. MODE 3: the product
+// MODE as above, and 5: MODE 0 with max(y, 0)^2 applied to the float32 sums (after the bias);
+// K a multiple of 64, at least 256; both matrices below 4 GiB. MODE 3: the product
 // of a narrow output with a long K (too few tiles to fill the card) summed in k_splits runs of K,
 // each run of every tile a work item of its own; the items write float32 planes of partial sums
 // [k_splits, M, N] that the next norm kernel adds up in their order.
@@ -517,6 +518,10 @@ __global__ __launch_bounds__(256) void gemm_wide_bf16_kernel(WideArgs a) {
           if (a.bias != nullptr && n < N)
             v[e] += a.bias_f32 ? ((const float*)a.bias)[n] : __bfloat162float(((const bf16_t*)a.bias)[n]);
           if (GROUPED) v[e] *= row_factor;
+          if (MODE == 5) {
+            const float r = fmaxf(v[e], 0.0f);
+            v[e] = r * r;
+          }
         }
       }
       *lo = w_pack_bf16(v[0], v[1]);
@@ -610,7 +615,7 @@ static int w_tiles(int mode, int M, int N) {
 
 // Does the wide-tile kernel take this product? Returns its number of tiles, or 0.
 CW_EXPORT int cw_gemm_bf16_wide_tiles(int mode, int M, int N, int K, int64_t ldx) {
-  if (M <= 0 || N <= 0 || (mode != 0 && mode != 2) || (mode == 2 && (N & 1))) return 0;
+  if (M <= 0 || N <= 0 || (mode != 0 && mode != 2 && mode != 5) || (mode == 2 && (N & 1))) return 0;
   if ((K & 63) || K < 256 || (ldx & 7) || ldx < K) return 0;
   if ((int64_t)N * K * 2 >= (1ll << 32) || (int64_t)M * ldx * 2 >= (1ll << 32)) return 0;
   return w_tiles(mode, M, N);
@@ -648,14 +653,15 @@ static int w_launch(WideArgs a, int workgroups, hipStream_t stream) {
 // units of the GPU (one workgroup fills a unit).
 CW_EXPORT int cw_gemm_bf16_wide(int mode, const void* X, int64_t ldx, const void* W, const void* bias, int bias_f32,
                                 void* C, int64_t ldc, int M, int N, int K, int workgroups, hipStream_t stream) {
-  if (M < 0 || N <= 0 || K <= 0 || (mode != 0 && mode != 2) || workgroups < 8) return CW_ERR_ARG;
+  if (M < 0 || N <= 0 || K <= 0 || (mode != 0 && mode != 2 && mode != 5) || workgroups < 8) return CW_ERR_ARG;
   if (((uintptr_t)X & 15) || ((uintptr_t)W & 15) || ((uintptr_t)C & 7)) return CW_ERR_ARG;
   if (mode == 2 && ((N & 1) || bias != nullptr)) return CW_ERR_ARG;
   if (ldc < (mode == 2 ? N / 2 : N)) return CW_ERR_ARG;
   if (M == 0) return CW_OK;
   if (cw_gemm_bf16_wide_tiles(mode, M, N, K, ldx) == 0) return CW_ERR_SIZE;
   WideArgs a{(const bf16_t*)X, ldx, (const bf16_t*)W, bias, bias_f32, C, ldc, M, N, K, 0, 0, 1};
-  return mode == 2 ? w_launch<2>(a, workgroups, stream) : w_launch<0>(a, workgroups, stream);
+  return mode == 2 ? w_launch<2>(a, workgroups, stream)
+                   : mode == 5 ? w_launch<5>(a, workgroups, stream) : w_launch<0>(a, workgroups, stream);
 }
 
 // parts[z] = x[:, run z of K] W[:, run z of K]^T for z < k_splits: float32 planes [k_splits, M, N]

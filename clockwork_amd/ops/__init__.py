@@ -1930,7 +1930,29 @@ def relu_squared_(x: torch.Tensor) -> torch.Tensor:
 
 
 def linear_relu_squared(x: torch.Tensor, weight: torch.Tensor, policy: "ProductPolicy | None" = None) -> torch.Tensor:
-    """max(x @ weight.T, 0)^2: the product, then the activation in place."""
+    """max(x @ weight.T, 0)^2. Few bfloat16 rows: the weight-streaming product with the activation
+    in its epilogue, applied to the float32 sums (one launch); else the product, then the
+    activation in place."""
+    _gpu(x, weight)
+    M, K = x.shape
+    N = weight.shape[0]
+    if (x.dtype == torch.bfloat16 and weight.dtype == torch.bfloat16 and weight.shape[1] == K and M <= STREAM_MAX_ROWS
+            and K % 8 == 0):
+        lib = _load("gemm")
+        if lib.cw_gemm_bf16_skinny_fast(5, M, N, K):
+            out = torch.empty((M, N), dtype=torch.bfloat16, device=x.device)
+            _check(lib.cw_gemm_bf16_skinny(5, _ptr(x), K, _ptr(weight), _ptr(out), N, M, N, K, 0, _stream()), "gemm_bf16_skinny(relu2)")
+            return out
+    # a long portion: the wide-tile kernel with the activation in its epilogue, from the sizes at
+    # which it takes the gate/up product of a gated feed-forward (the same kernel, the same gain)
+    if (x.dtype == torch.bfloat16 and weight.dtype == torch.bfloat16 and weight.shape[1] == K and M >= WIDE_SWIGLU_MIN_ROWS
+            and x.stride(1) == 1 and x.stride(0) % 8 == 0 and weight.is_contiguous()):
+        lib = _load("gemm_tile")
+        if lib.cw_gemm_bf16_wide_tiles(5, M, N, K, x.stride(0)) >= WIDE_SWIGLU_MIN_TILES:
+            out = torch.empty((M, N), dtype=torch.bfloat16, device=x.device)
+            _check(lib.cw_gemm_bf16_wide(5, _ptr(x), x.stride(0), _ptr(weight), None, 0, _ptr(out), N, M, N, K,
+                                         _compute_units(x.device), _stream()), "gemm_bf16_wide(relu2)")
+            return out
     return relu_squared_(linear(x, weight, policy=policy))
 
 

@@ -70,7 +70,9 @@ class GatedMLP(Part):
 class DenseMLP(Part):
     """down(act(up(x))) (``DenseMLPSpec``). "gelu": the up product with the erf GELU (float32
     inside) in its epilogue for few rows, as a kernel of its own behind the product otherwise;
-    "relu2": the product, then max(z, 0)^2 in place; the down product."""
+    "relu2": max(z, 0)^2 on the float32 sums in the epilogue of the up product for few rows
+    (the weight-streaming kernel) and for long portions (the wide-tile kernel), in place behind
+    the product otherwise; the down product."""
 
     graph_safe = True
 

@@ -84,6 +84,19 @@ def test_squared_relu_feed_forward(dtype, hidden, rows):
     x = torch.randn(rows, hidden, generator=torch.Generator().manual_seed(3)).to(dtype)
     got = part.forward(x.to(DEV), SimpleNamespace()).double().cpu()
     close(got, plain.dense_feed_forward(x.double(), {"up": w["up_weight"], "down": w["down_weight"]}, ""), dtype)
+    if dtype == torch.bfloat16 and rows == 200:
+        # the same activation in the epilogues of the up product: of the weight-streaming kernel
+        # (few rows) and of the wide-tile kernel (a long portion of a wide layer), against the
+        # product followed by the activation kernel
+        for m, k, n in [(5, 256, 8704), (40, 512, 8704), (1100, 256, 8704), (1030, 320, 8650)]:
+            gen = torch.Generator().manual_seed(m)
+            a = torch.randn(m, k, generator=gen).to(dtype).to(DEV)
+            wt = (torch.randn(n, k, generator=gen) / k ** 0.5).to(dtype).to(DEV)
+            want = torch.relu(a.double() @ wt.double().t()).square().cpu()
+            scale = float(want.square().mean().sqrt())
+            for got in (ops.linear_relu_squared(a, wt), ops.relu_squared_(ops.linear(a, wt))):
+                # squares reach far above their scale: an element is held to its own size
+                assert bool(((got.double().cpu() - want).abs() <= 1.5e-2 * want.abs() + 1e-2 * scale).all())
     z = torch.tensor([-3.0, -0.0, 0.0, 0.5, 2.0, 64.0]).to(dtype).to(DEV)
     torch.testing.assert_close(ops.relu_squared_(z).float().cpu(), torch.tensor([0.0, 0.0, 0.0, 0.25, 4.0, 4096.0]))
 
