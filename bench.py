@@ -575,11 +575,11 @@ def nenodra_config(size: dict, layers: int, max_positions: int) -> dict:
     rot = {"base": 10000.0, "dims": 64}
     gated = {"heads": size["heads"], "kv_heads": size["kv_heads"], "dim": size["head_dim"], "vdim": size["head_dim"],
              "scale": size["head_dim"] ** -0.5, "mask": {"size": size["window"]}, "rot": rot}
-    two_map = {"heads": size["heads"], "kv_heads": size["kv_heads"], "dim": size["dim"], "vdim": size["vdim"], "diff": 0.5,
+    two_map = {"heads": size["heads"], "kv_heads": size["kv_heads"], "dim": size["dim"], "vdim": size["vdim"], "diff": 0.4,
                "scale": size["dim"] ** -0.5, "mask": {"size": size["window"]}, "rot": rot}
     kinds = [("attention_2", gated, dense), ("attention", two_map, routed), ("attention", two_map, dense), ("attention_2", gated, routed)]
-    return {"architecture": "Nenodra", "vocab": DESIGN_VOCAB, "width": size["width"], "residual_mult": 0.5, "logit_scale": 0.5,
-            "norm": {"eps": 1e-6},
+    return {"architecture": "Nenodra", "vocab": DESIGN_VOCAB, "width": size["width"], "residual_mult": 0.6, "logit_scale": 0.25,
+            "norm": {"eps": 1e-5},
             "layers": [{"type": kinds[i % 4][0], "mixer": kinds[i % 4][1], "mlp": kinds[i % 4][2]} for i in range(layers)]}
 
 

@@ -810,6 +810,94 @@ __global__ __launch_bounds__(1024) void headnorm_rope_store_kernel(
   }
 }
 
+// The same for bfloat16 vectors of 8, 16, ... 512 elements whose rotated part is a multiple of 16:
+// a lane holds 8 neighbouring elements of a vector (one 16-byte load and store), dim / 8 lanes a
+// vector, several vectors a wave. The sum of squares meets over the vector's lanes by exchanges;
+// a rotated element's partner, dims / 2 elements away, lies in the lane dims / 16 further.
+// Element by element the arithmetic is the kernel's above.
+typedef __attribute__((ext_vector_type(4))) unsigned int cw_u32x4_t;
+template <typename WT, typename BT>
+__global__ __launch_bounds__(256) void headnorm_rope_store_vec_kernel(
+    bf16_t* __restrict__ proj, int64_t stride, int q_off, int k_off, int v_off, int nqv, int nkv, int dim, int nv,
+    const BT* __restrict__ bias, const WT* __restrict__ qw, const WT* __restrict__ kw, float eps,
+    const int* __restrict__ positions, const float* __restrict__ freq, int rdims, const int* __restrict__ slots,
+    bf16_t* __restrict__ k_plane, bf16_t* __restrict__ v_plane, int v_from_keys, int64_t cache_rows) {
+  extern __shared__ float hn_vals[];  // the token's cosines and sines [2][rdims / 2]
+  const int64_t t = blockIdx.x;
+  bf16_t* row = proj + t * stride;
+  int64_t slot = slots ? (int64_t)slots[t] : -1;
+  if (slot >= cache_rows) slot = -1;
+  const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
+  if (slot >= 0 && v_plane) {
+    const int src = v_from_keys ? k_off : v_off;
+    bf16_t* vd = v_plane + slot * nv;
+    for (int j = threadIdx.x; j < nv; j += 256)
+      vd[j] = __float2bfloat16(__bfloat162float(row[src + j]) + (bias ? cw_to_float(bias[src + j]) : 0.0f));
+  }
+  const float pos = positions ? (float)positions[t] : 0.0f;
+  const int half = rdims / 2;
+  float* cosines = hn_vals;
+  float* sines = cosines + half;
+  for (int i = threadIdx.x; i < half; i += 256) sincosf(pos * freq[i], &sines[i], &cosines[i]);
+  __syncthreads();
+  const int lanes = dim >> 3, per_wave = 64 / lanes;   // lanes of a vector (a power of two), vectors of a wave
+  const int sub = lane & (lanes - 1), j0 = sub * 8;
+  const bool rotated = j0 < rdims, low = j0 < half;
+  const int partner = rotated ? (low ? lane + (half >> 3) : lane - (half >> 3)) : lane;
+  const int n_vec = nqv + nkv;
+  for (int first = 0; first < n_vec; first += 4 * per_wave) {  // every lane of a wave stays for the exchanges
+    const int vec = first + wave * per_wave + lane / lanes;
+    const bool is_q = vec < nqv;
+    const bool live = vec < n_vec && (is_q || slot >= 0);
+    const int base = (is_q ? q_off + vec * dim : k_off + (vec - nqv) * dim) + j0;
+    const WT* w = is_q ? qw : kw;
+    float v[8];
+#pragma unroll
+    for (int i = 0; i < 8; ++i) v[i] = 0.0f;
+    if (live) {
+      const cw_u32x4_t raw = *reinterpret_cast<const cw_u32x4_t*>(row + base);
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        v[2 * i] = cw_bf16_bits_to_float((uint16_t)(raw[i] & 0xffffu));
+        v[2 * i + 1] = cw_bf16_bits_to_float((uint16_t)(raw[i] >> 16));
+      }
+      if (bias) {
+#pragma unroll
+        for (int i = 0; i < 8; ++i) v[i] += cw_to_float(bias[base + i]);
+      }
+    }
+    float ss = 0.0f;
+#pragma unroll
+    for (int i = 0; i < 8; ++i) ss += v[i] * v[i];
+    for (int off = 1; off < lanes; off <<= 1) ss += __shfl_xor(ss, off, 64);
+    const float inv = w ? 1.0f / sqrtf(ss / (float)dim + eps) : 1.0f;
+    float pv[8];
+#pragma unroll
+    for (int i = 0; i < 8; ++i) pv[i] = __shfl(v[i], partner, 64);
+    if (!live) continue;
+    uint16_t o[8];
+#pragma unroll
+    for (int i = 0; i < 8; ++i) {
+      float r;
+      if (rotated) {
+        const int idx = (low ? j0 : j0 - half) + i;
+        const float a = (low ? v[i] : pv[i]) * inv * (w ? cw_to_float(w[idx]) : 1.0f);
+        const float b = (low ? pv[i] : v[i]) * inv * (w ? cw_to_float(w[idx + half]) : 1.0f);
+        const float sn = sines[idx], c = cosines[idx];
+        r = low ? a * c - b * sn : b * c + a * sn;
+      } else {
+        r = v[i] * inv * (w ? cw_to_float(w[j0 + i]) : 1.0f);
+      }
+      o[i] = cw_float_to_bf16_bits(r);
+    }
+    cw_u32x4_t packed;
+#pragma unroll
+    for (int i = 0; i < 4; ++i) packed[i] = (uint32_t)o[2 * i] | ((uint32_t)o[2 * i + 1] << 16);
+    bf16_t* dst = is_q ? row + base : k_plane + slot * ((int64_t)nkv * dim) + (int64_t)(vec - nqv) * dim + j0;
+    *reinterpret_cast<cw_u32x4_t*>(dst) = packed;
+  }
+}
+
 CW_EXPORT int cw_headnorm_rope_store(void* proj, int dtype, int64_t stride, int q_off, int k_off, int v_off, int nqv, int nkv,
                                      int dim, int nv, const void* bias, int b_dtype, const void* qw, const void* kw,
                                      int w_dtype, float eps, const int* positions, const float* freq, int rdims,
@@ -823,6 +911,23 @@ CW_EXPORT int cw_headnorm_rope_store(void* proj, int dtype, int64_t stride, int 
   if (!proj || (rdims && (!freq || !positions)) || (slots && nkv && !k_plane) || (slots && nv && !v_plane)) return CW_ERR_ARG;
   if ((qw == nullptr) != (kw == nullptr)) return CW_ERR_ARG;
   if (T == 0) return CW_OK;
+  // bfloat16 vectors that lanes of 8 elements tile: the kernel of 16-byte accesses
+  if (dtype == CW_BF16 && dim >= 8 && dim <= 512 && !(dim & (dim - 1)) && !(rdims & 15) && !(q_off & 7) && !(k_off & 7) &&
+      !(stride & 7) && !((uintptr_t)proj & 15) && !((uintptr_t)k_plane & 15)) {
+    const size_t lds_vec = (size_t)(rdims ? rdims : 2) * sizeof(float);
+#define CW_LAUNCH_VEC(WT_, BT_)                                                                                         \
+  hipLaunchKernelGGL((headnorm_rope_store_vec_kernel<WT_, BT_>), dim3(T), dim3(256), lds_vec, stream, (bf16_t*)proj, stride, \
+                     q_off, k_off, v_off, nqv, nkv, dim, nv, (const BT_*)bias, (const WT_*)qw, (const WT_*)kw, eps, positions, \
+                     freq, rdims, slots, (bf16_t*)k_plane, (bf16_t*)v_plane, v_from_keys, cache_rows)
+    const int wt_v = qw ? w_dtype : CW_BF16, bt_v = bias ? b_dtype : CW_BF16;
+    if (wt_v == CW_BF16 && bt_v == CW_BF16) CW_LAUNCH_VEC(bf16_t, bf16_t);
+    else if (wt_v == CW_F32 && bt_v == CW_BF16) CW_LAUNCH_VEC(float, bf16_t);
+    else if (wt_v == CW_BF16 && bt_v == CW_F32) CW_LAUNCH_VEC(bf16_t, float);
+    else if (wt_v == CW_F32 && bt_v == CW_F32) CW_LAUNCH_VEC(float, float);
+    else return CW_ERR_DTYPE;
+#undef CW_LAUNCH_VEC
+    return cw_launch_status();
+  }
   // a wave a vector at a time: as many waves as there are vectors, 4 to 16
   const int n_vec = nqv + nkv;
   int waves = n_vec < 4 ? 4 : n_vec > 16 ? 16 : n_vec;

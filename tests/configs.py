@@ -245,7 +245,7 @@ NENODRA_A = {
 NENODRA_B = {
     "architecture": "Nenodra", "vocab": 127, "width": 100, "residual_mult": 1.0, "logit_scale": 1.0, "norm": {"eps": 3e-4},
     "layers": [
-        _nenodra_two_map(3, 1, 40, 24, 0.16, 0.5, 300, 250000.0, 2, (50, 2, 1)),
+        _nenodra_two_map(3, 1, 40, 24, 0.16, 0.45, 300, 200000.0, 2, (50, 2, 1)),
         _nenodra_gated(5, 5, 12, 0.3, 1, 50.0, 12, 130),
         _nenodra_two_map(2, 1, 8, 32, 0.35, 0.1, 40, 10.0, 0, (36, 7, 4)),
     ],
