@@ -2,7 +2,7 @@
 // ``experts`` small gated feed-forwards, chosen by a router.
 //
 //   1. moe_route:  z = router x in float32, r = 1 / (1 + exp(-z)) (or softmax over the experts),
-//                  the ``top`` largest r (the lower index first among equals), optionally
+//                  the ``top`` largest r, chosen by their z (the lower index first among equals), optionally
 //                  divided by their sum. One workgroup a token.
 //   2. moe_plan:   the (token, choice) pairs sorted by expert into rows; every expert's rows begin
 //                  at a multiple of MOE_TILE_ROWS, so a tile of rows belongs to one expert. One
@@ -41,7 +41,8 @@ template <typename T>
 __global__ __launch_bounds__(256) void moe_route_kernel(const T* __restrict__ x, const T* __restrict__ router, int H, int E,
                                                         int top, int kind, int* __restrict__ choice,
                                                         float* __restrict__ score) {
-  __shared__ float r[MOE_MAX_EXPERTS];
+  __shared__ float r[MOE_MAX_EXPERTS];  // logits, then scores
+  __shared__ float z[MOE_MAX_EXPERTS];  // logits
   const int64_t t = blockIdx.x;
   const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
   const T* xr = x + t * H;
@@ -75,6 +76,9 @@ __global__ __launch_bounds__(256) void moe_route_kernel(const T* __restrict__ x,
   }
   __syncthreads();
   if (wave != 0) return;
+  // the choice is made on the logits, which order the experts as the scores do and still tell
+  // apart two experts whose scores both round to 1
+  for (int e = lane; e < E; e += 64) z[e] = r[e];
   if (kind == MOE_ROUTER_SOFTMAX) {
     float m = -3.0e38f;
     for (int e = lane; e < E; e += 64) m = fmaxf(m, r[e]);
@@ -87,11 +91,11 @@ __global__ __launch_bounds__(256) void moe_route_kernel(const T* __restrict__ x,
     for (int e = lane; e < E; e += 64) r[e] = 1.0f / (1.0f + expf(-r[e]));
   }
   for (int k = 0; k < top; ++k) {
-    // the largest score still there; among equals the lowest index
-    float best = -1.0f;
+    // the largest logit still there; among equals the lowest index
+    float best = -3.4e38f;
     int at = 0x7fffffff;
     for (int e = lane; e < E; e += 64)
-      if (r[e] > best) { best = r[e]; at = e; }
+      if (z[e] > best) { best = z[e]; at = e; }
 #pragma unroll
     for (int off = 32; off > 0; off >>= 1) {
       const float ob = __shfl_xor(best, off, 64);
@@ -99,9 +103,11 @@ __global__ __launch_bounds__(256) void moe_route_kernel(const T* __restrict__ x,
       if (ob > best || (ob == best && oa < at)) { best = ob; at = oa; }
     }
     if (lane == 0) {
+      const bool found = at < E;   // not so if the logits are no numbers: a row that holds no token
+      if (!found) at = k < E ? k : E - 1;
       choice[t * top + k] = at;
-      score[t * top + k] = best;
-      r[at] = -2.0f;  // scores are not negative: never chosen again
+      score[t * top + k] = found ? r[at] : 0.0f;
+      if (found) z[at] = -3.4e38f;  // never chosen again
     }
   }
 }

@@ -381,7 +381,8 @@ class RoutedExpertsSpec:
     """A feed-forward made of ``num_experts`` small gated ones, E(u) = down(silu(gate u) * (up u)),
     no biases, of which every token uses ``top_k``: r = ``router``(W_r x) in float32 ("sigmoid":
     the logistic function of each logit by itself; "softmax": over the experts), the top_k
-    largest r chosen (the lower index first among equals), divided by their sum if
+    largest r chosen (compared through their logits, which still differ where two r round to 1;
+    the lower index first among equals), divided by their sum if
     ``renormalize``. ``weight_on`` "input": the result is the sum of E_e(r_e x); "output": the sum
     of r_e E_e(x)."""
 
