@@ -272,3 +272,39 @@ NENODRA_LONG = {
 }
 # name -> (config, weight seed, cache block size)
 NENODRA_CONFIGS = {"NA": (NENODRA_A, 41, 8), "NB": (NENODRA_B, 42, 16), "NC": (NENODRA_C, 43, 4)}
+
+
+def random_nenodra_config(seed: int) -> dict:
+    """A model of the design drawn at random: three to seven layers that share nothing, head sizes
+    that the matrix-core kernels take and ones they do not, windows shorter and longer than a
+    page, rotation of all, a part and nothing, one to four experts a token, layers without a
+    feed-forward."""
+    import random
+
+    rng = random.Random(seed)
+    layers = []
+    for _ in range(rng.randint(3, 7)):
+        kv = rng.choice([1, 2, 4])
+        heads = kv * rng.choice([1, 2, 3, 4])
+        dim = rng.choice([16, 24, 32, 40, 48, 64, 80, 96, 128])
+        rot = rng.choice([dim, dim // 4 * 2, 16, 0, dim])
+        scale = dim ** -0.5 * rng.choice([0.5, 1.0, 2.0])
+        window = rng.choice([1, 33, 64, 65, 100, 130, 200, 257])
+        base = rng.choice([100.0, 10000.0, 5e5])
+        kind = rng.choice(["dense", "dense", "moe", "moe", "moe", None])
+        if kind == "dense":
+            mlp = rng.choice([72, 104, 200, 512])
+        elif kind == "moe":
+            experts = rng.choice([2, 4, 5, 8, 16])
+            mlp = (rng.choice([40, 64, 88, 128, 256]), experts, rng.randint(1, min(4, experts)))
+        else:
+            mlp = None
+        if rng.random() < 0.5:
+            layers.append(_nenodra_two_map(heads, kv, dim, rng.choice([16, 32, 48, 64, 96, 128]), scale, rng.choice([0.2, 0.45, 0.8]),
+                                           window, base, rot, mlp))
+        else:
+            layers.append(_nenodra_gated(heads, kv, dim, scale, window, base, rot, mlp))
+    return {"architecture": "Nenodra", "vocab": rng.choice([300, 500, 1000]), "width": rng.choice([128, 192, 320, 384, 512]),
+            "residual_mult": rng.choice([0.3, 0.6, 1.0]), "logit_scale": rng.choice([0.25, 0.7, 2.0]),
+            "norm": {"eps": rng.choice([1e-6, 1e-5])}, "layers": layers}
+

@@ -610,6 +610,48 @@ def test_models_in_four_batching_modes(nenodra_dirs, name, mode, dtype):
     assert all(p.num_free == runner.manager.num_blocks for p in runner.manager.pools)
 
 
+@pytest.mark.parametrize("seed", range(2000, 2010))
+def test_models_drawn_at_random(tmp_path, seed):
+    """Ten models whose sizes, layer order and constants are drawn at random, six requests of 1 to
+    420 tokens on pages of 64 barely enough for four of them, as mixed batches, in portions and as
+    prefill then single tokens. float32 against the plain implementation as the model stands (its
+    routers scaled down, so that no logit lies where the logistic function is flat and few choices
+    are close calls); bfloat16 with the routed layers made dense, because a rounded router input
+    flips close choices, which a comparison of logits cannot tell from a fault."""
+    import copy
+    import random
+
+    from safetensors.torch import load_file, save_file
+
+    from clockwork_amd.weights.random_init import write_random_model
+    from tests.configs import random_nenodra_config
+
+    cfg = random_nenodra_config(seed)
+    dense = copy.deepcopy(cfg)
+    for entry in dense["layers"]:
+        if entry["mlp"] is not None and entry["mlp"]["kind"] == "moe":
+            entry["mlp"] = {"kind": "dense", "ff": 2 * entry["mlp"]["expert"]["ff"]}
+    rng = random.Random(seed)
+    lengths = [rng.randint(100, 420), rng.randint(2, 90), rng.randint(200, 330), rng.randint(40, 300), 1, 65]
+    for dtype, config in (("float32", cfg), ("bfloat16", dense)):
+        model_dir = write_random_model(tmp_path / dtype, config, seed)
+        path = str(Path(model_dir) / "model.safetensors")
+        tensors = load_file(path)
+        for key in tensors:
+            if key.endswith("mlp.router"):
+                tensors[key] = (tensors[key].float() * 0.05).to(tensors[key].dtype)
+        save_file(tensors, path)
+        requests = _requests(config["vocab"], lengths, seed)
+        oracle = plain.PlainNenodra(model_dir)
+        ref = {rid: oracle.logits(toks) for rid, toks in requests.items()}
+        for mode in ("mixed", "portions", "prefill_then_decode"):
+            runner = replay.make_runner(model_dir, dtype, 64, replay.pages_needed(requests, 4, 64) + 1)
+            got = replay.run_trace(runner, getattr(replay, mode)(requests))
+            assert len(got) == sum(len(t) for t in requests.values())
+            _check(got, ref, dtype)
+            assert not runner.manager.live_requests()
+
+
 def test_the_stream_after_every_layer(nenodra_dirs):
     """Float32, one request: the residual stream after every layer against the plain implementation's."""
     cfg, _, block_size = NENODRA_CONFIGS["NA"]
