@@ -58,6 +58,11 @@ class GroupLayout:
         return getattr(self.need, "segment", None) if self.is_kv else None
 
     @property
+    def keep_first(self) -> int:
+        """Positions at a request's start that every later token reads, window or not."""
+        return int(getattr(self.need, "keep_first", 0) or 0) if self.is_kv else 0
+
+    @property
     def keeps_all(self) -> bool:
         """Does a request keep every page of the group until it ends?"""
         return self.window is None and self.segment is None
@@ -303,7 +308,9 @@ class CacheManager:
             if self.kv_groups[g].keeps_all:
                 continue
             first = min(self._first_needed_block(g, computed), len(rec.tables[g]))
-            for b in range(rec.released[g], first):
+            # the pages of the first positions that stay readable are never given back
+            kept = self._blocks_for(self.kv_groups[g].keep_first)
+            for b in range(max(rec.released[g], kept), first):
                 page = rec.tables[g][b]
                 if page != NO_PAGE:
                     pool.drop(page)

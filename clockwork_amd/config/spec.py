@@ -68,11 +68,14 @@ class PagedRowsSpec:
     tables and slots of its group. ``segment`` S (instead of a window): positions are cut into
     segments of S counted from 0 and a token reads the earlier tokens of its own segment only;
     pages wholly before the segment of the next token are given back while the request runs.
+    ``keep_first`` n (with a window): every later token also reads the request's first n positions,
+    so the pages that hold them stay with the request until it ends.
     """
 
     planes: tuple
     window: Optional[int] = None
     segment: Optional[int] = None
+    keep_first: int = 0
 
     def __post_init__(self):
         names = [name for name, _ in self.planes]
@@ -85,9 +88,13 @@ class PagedRowsSpec:
             raise ValueError("a paged cache has a window or segments, not both")
         if self.segment is not None and self.segment < 1:
             raise ValueError(f"segment must be positive, got {self.segment}")
+        if self.keep_first < 0 or (self.keep_first and self.window is None):
+            raise ValueError("first positions are kept readable behind a window only, and their number is not negative")
 
     def group_key(self) -> tuple:
         key = ("rows", tuple((name, tuple(shape)) for name, shape in self.planes), self.window)
+        if self.keep_first:
+            key = key + (("keep_first", self.keep_first),)
         return key if self.segment is None else key + (("segment", self.segment),)
 
 
@@ -170,11 +177,14 @@ class RunEntry:
     (what the embedding part made of the step's tokens) is added to the residual stream once
     more right before this entry's block (a repeated run of layers that is fed the input again
     at every pass); the block's first norm must be able to add it (``accepts_stream_input``).
+    ``reenter`` n: right before this entry's block the stream is made anew from itself and the
+    model's input by the model's re-entry part (``ModelSpec.reentry``), as pass number n.
     """
 
     layer: int
     cache_from: Optional[int] = None
     add_input: bool = False
+    reenter: Optional[int] = None
 
 
 @dataclass
@@ -195,6 +205,9 @@ class ModelSpec:
     # the longest request the model can run (a learned position table ends there); None: no limit
     # of the model's own
     max_positions: Optional[int] = None
+    # spec of the part that makes the stream anew from itself and the model's input before the run
+    # entries that say ``reenter`` (the passes of a repeated run of layers); None: no such entries
+    reentry: Any = None
     # free-form facts for reporting (bench config lines and the like), never read by parts
     info: dict = field(default_factory=dict)
 
@@ -211,6 +224,8 @@ class ModelSpec:
                     raise ValueError(f"run[{i}].cache_from={entry.cache_from} must name an earlier entry")
                 if self.run[entry.cache_from].cache_from is not None:
                     raise ValueError(f"run[{i}].cache_from names an entry that itself borrows a cache")
+            if entry.reenter is not None and self.reentry is None:
+                raise ValueError(f"run[{i}] re-enters the stream, but the model has no re-entry part")
 
 
 @dataclass(frozen=True)

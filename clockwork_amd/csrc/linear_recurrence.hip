@@ -4,6 +4,16 @@
 // z_t = A2 u_t + b (u_t the token's ``rank`` inputs). o_t is optionally RMS-normed over vdim
 // with a weight shared by the heads and multiplied by silu(g_t).
 //
+// Variants (LinRecForm), for a recurrence of another family:
+//   decay_kind 1:  a_t = exp(-exp(z_t)) with z_t = A2 tanh(u_t) + b.
+//   bonus [heads, dim]:  the output reads the state BEFORE the token joins it, and the token itself
+//                  through the bonus:  o_t = (S_(t-1) + diag(bonus) k_t v_t^T)^T q_t,  then
+//                  S_t = diag(a_t) S_(t-1) + k_t v_t^T.
+//   norm_w_stride: vdim when every head has norm weights of its own ([heads, vdim]), else 0.
+//   u, u_stride:   the decay input as rows of a tensor of its own (else columns of proj).
+// q, k, v and the gate may also lie in planes one behind the other, [4][T, heads * dim]: then
+// stride is the plane's row and an offset a multiple of the plane's size.
+//
 // A workgroup owns one (request, head): the state lives in registers for the whole portion (a
 // thread holds a run of rows of one column), tokens are walked in order, sixteen at a time: their
 // q, k, v and decays are staged in LDS, the walk itself has no barrier, the outputs' partial sums
@@ -12,6 +22,22 @@
 #include "common.h"
 
 #define LR_TC 16  // tokens staged at a time
+
+struct LinRecForm {
+  int decay_kind;        // 0: sigmoid(z)^(1/tau); 1: exp(-exp(z)) with tanh on the decay input
+  const float* bonus;    // [heads, dim] or null
+  int norm_w_stride;     // 0 or vdim
+  const void* u;         // decay input rows, or null: columns u_off .. of proj
+  int64_t u_stride;
+  int state_stride;      // floats between two slots' states (>= heads * dim * vdim)
+};
+
+__device__ __forceinline__ float lr_decay(float z, int kind, float inv_tau) {
+  if (kind == 1) return expf(-expf(z));
+  // log(sigmoid(z)) without cancellation, then the 1/tau-th power
+  const float ls = z < 0.0f ? z - log1pf(expf(z)) : -log1pf(expf(-z));
+  return expf(ls * inv_tau);
+}
 
 struct LinRecParams {
   const void* proj;   // [T, stride]: a token's q (heads * dim at q_off), k (k_off), v (heads * vdim at v_off),
@@ -29,7 +55,7 @@ struct LinRecParams {
 };
 
 template <typename T, int RPT>
-__global__ __launch_bounds__(256) void linear_recurrence_kernel(LinRecParams p) {
+__global__ __launch_bounds__(256) void linear_recurrence_kernel(LinRecParams p, LinRecForm f) {
   extern __shared__ __align__(16) float smem[];
   const int D = p.dim, V = p.vdim, Hn = p.heads;
   const int r = blockIdx.x, h = blockIdx.y, tid = threadIdx.x;
@@ -48,9 +74,13 @@ __global__ __launch_bounds__(256) void linear_recurrence_kernel(LinRecParams p) 
   float* part = vs + LR_TC * V;     // [TC][DS][V]
 
   float S[RPT];
-  float* st = p.state + (((int64_t)slot * Hn + h) * D) * V;
+  float* st = p.state + (int64_t)slot * f.state_stride + ((int64_t)h * D) * V;
+  float bonus[RPT];
 #pragma unroll
-  for (int rr = 0; rr < RPT; ++rr) S[rr] = (active && d0 + rr < D) ? st[(int64_t)(d0 + rr) * V + v] : 0.0f;
+  for (int rr = 0; rr < RPT; ++rr) {
+    S[rr] = (active && d0 + rr < D) ? st[(int64_t)(d0 + rr) * V + v] : 0.0f;
+    bonus[rr] = (f.bonus && active && d0 + rr < D) ? f.bonus[h * D + d0 + rr] : 0.0f;
+  }
 
   const T* proj = (const T*)p.proj;
   const T* a2 = (const T*)p.a2;
@@ -65,10 +95,13 @@ __global__ __launch_bounds__(256) void linear_recurrence_kernel(LinRecParams p) 
       ks[idx] = cw_to_float(row[p.k_off + h * D + d]);
       float z = p.a2b ? p.a2b[h * D + d] : 0.0f;
       const T* w = a2 + (int64_t)(h * D + d) * p.rank;
-      for (int c = 0; c < p.rank; ++c) z += cw_to_float(w[c]) * cw_to_float(row[p.u_off + c]);
-      // log(sigmoid(z)) without cancellation, then the 1/tau-th power
-      const float ls = z < 0.0f ? z - log1pf(expf(z)) : -log1pf(expf(-z));
-      as[idx] = expf(ls * p.inv_tau);
+      const T* u = f.u ? (const T*)f.u + (int64_t)(row0 + t0 + t) * f.u_stride : row + p.u_off;
+      if (f.decay_kind == 1) {
+        for (int c = 0; c < p.rank; ++c) z += cw_to_float(w[c]) * tanhf(cw_to_float(u[c]));
+      } else {
+        for (int c = 0; c < p.rank; ++c) z += cw_to_float(w[c]) * cw_to_float(u[c]);
+      }
+      as[idx] = lr_decay(z, f.decay_kind, p.inv_tau);
     }
     for (int idx = tid; idx < nt * V; idx += 256) {
       const int t = idx / V, c = idx - t * V;
@@ -83,8 +116,10 @@ __global__ __launch_bounds__(256) void linear_recurrence_kernel(LinRecParams p) 
         for (int rr = 0; rr < RPT; ++rr) {
           const int d = d0 + rr;
           if (d < D) {
-            S[rr] = as[t * D + d] * S[rr] + ks[t * D + d] * vv;
-            po += qs[t * D + d] * S[rr];
+            const float kv = ks[t * D + d] * vv;
+            if (f.bonus) po += qs[t * D + d] * (S[rr] + bonus[rr] * kv);
+            S[rr] = as[t * D + d] * S[rr] + kv;
+            if (!f.bonus) po += qs[t * D + d] * S[rr];
           }
         }
         part[(t * DS + s) * V + v] = po;
@@ -113,7 +148,7 @@ __global__ __launch_bounds__(256) void linear_recurrence_kernel(LinRecParams p) 
         const int c = lane + u * 64;
         if (c < V) {
           float val = o[u] * inv;
-          if (p.norm_w) val *= p.norm_w[c];
+          if (p.norm_w) val *= p.norm_w[h * f.norm_w_stride + c];
           if (p.g_off >= 0) {
             const float g = cw_to_float(proj[trow * p.stride + p.g_off + h * V + c]);
             val *= g / (1.0f + expf(-g));
@@ -141,13 +176,18 @@ CW_EXPORT int cw_linear_recurrence(int dtype, const void* proj, int64_t stride, 
                                    int u_off, const void* a2, const float* a2b, const float* norm_w, float* state,
                                    int n_slots, const int* state_slots, const int* cu_q, void* out, int n_requests,
                                    int heads, int dim, int vdim, int rank, float q_scale, float inv_tau, float eps,
-                                   hipStream_t stream) {
+                                   int decay_kind, const float* bonus, int norm_w_stride, const void* u, int64_t u_stride,
+                                   int64_t state_stride, hipStream_t stream) {
   if (n_requests < 0 || !proj || !a2 || !state || !state_slots || !cu_q || !out) return CW_ERR_ARG;
-  if (heads <= 0 || rank <= 0 || n_slots <= 0 || q_off < 0 || k_off < 0 || v_off < 0 || u_off < 0) return CW_ERR_ARG;
-  if (q_off + heads * dim > stride || k_off + heads * dim > stride || v_off + heads * vdim > stride ||
-      u_off + rank > stride || (g_off >= 0 && g_off + heads * vdim > stride))
+  if (heads <= 0 || rank <= 0 || n_slots <= 0 || q_off < 0 || k_off < 0 || v_off < 0 || u_off < 0 || stride <= 0) return CW_ERR_ARG;
+  if (q_off % stride + heads * dim > stride || k_off % stride + heads * dim > stride || v_off % stride + heads * vdim > stride ||
+      (!u && u_off + rank > stride) || (g_off >= 0 && g_off % stride + heads * vdim > stride))
+    return CW_ERR_ARG;
+  if (decay_kind < 0 || decay_kind > 1 || (norm_w_stride != 0 && norm_w_stride != vdim) || (u && u_stride < rank) ||
+      state_stride < (int64_t)heads * dim * vdim || state_stride > 0x7fffffff)
     return CW_ERR_ARG;
   if (!cw_linear_recurrence_supported(dim, vdim)) return CW_ERR_SIZE;
+  const LinRecForm form = {decay_kind, bonus, norm_w_stride, u, u_stride, (int)state_stride};
   if (n_requests == 0) return CW_OK;
   if (heads > 65535) return CW_ERR_SIZE;
   LinRecParams p;
@@ -164,7 +204,7 @@ CW_EXPORT int cw_linear_recurrence(int dtype, const void* proj, int64_t stride, 
     if (smem > 48 * 1024 && hipFuncSetAttribute((const void*)linear_recurrence_kernel<T_, RPT_>,                   \
                                                 hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem) != hipSuccess) \
       return CW_ERR_LAUNCH;                                                                                        \
-    hipLaunchKernelGGL((linear_recurrence_kernel<T_, RPT_>), grid, block, smem, stream, p);                        \
+    hipLaunchKernelGGL((linear_recurrence_kernel<T_, RPT_>), grid, block, smem, stream, p, form);                        \
   } while (0)
 #define CW_BY_ROWS(T_)                         \
   do {                                         \
@@ -225,6 +265,7 @@ struct SegParams {
   int heads, dim, vdim, rank, n_slots, n_tokens;
   float q_scale, inv_tau, eps;
   int seg_tokens;         // the most tokens a segment has
+  LinRecForm form;
 };
 
 template <typename T> struct LrVec;
@@ -252,15 +293,17 @@ __global__ __launch_bounds__(256) void lrs_prepare_kernel(SegParams p) {
   const T* proj = (const T*)p.proj;
   const T* a2 = (const T*)p.a2;
   constexpr int N = LrVec<T>::N;
-  const bool vec = p.rank % N == 0 && p.u_off % N == 0 && p.stride % N == 0 && !((uintptr_t)proj & 15) && !((uintptr_t)a2 & 15);
+  const bool vec = !p.form.u && p.rank % N == 0 && p.u_off % N == 0 && p.stride % N == 0 && !((uintptr_t)proj & 15) && !((uintptr_t)a2 & 15);
   for (int64_t idx = (int64_t)blockIdx.x * 256 + threadIdx.x; idx < n; idx += (int64_t)gridDim.x * 256) {
     const int64_t t = idx / HD;
     const int c = (int)(idx - t * HD);
     const T* row = proj + t * p.stride;
     float z = p.a2b ? p.a2b[c] : 0.0f;
     const T* w = a2 + (int64_t)c * p.rank;
-    const T* u = row + p.u_off;
-    if (vec) {  // 16 bytes of the decay matrix's row and of the token's decay input at a time
+    const T* u = p.form.u ? (const T*)p.form.u + t * p.form.u_stride : row + p.u_off;
+    if (p.form.decay_kind == 1) {
+      for (int e = 0; e < p.rank; ++e) z += cw_to_float(w[e]) * tanhf(cw_to_float(u[e]));
+    } else if (vec) {  // 16 bytes of the decay matrix's row and of the token's decay input at a time
       for (int e = 0; e < p.rank; e += N) {
         float wv[N], uv[N];
         LrVec<T>::load(w + e, wv);
@@ -271,8 +314,7 @@ __global__ __launch_bounds__(256) void lrs_prepare_kernel(SegParams p) {
     } else {
       for (int e = 0; e < p.rank; ++e) z += cw_to_float(w[e]) * cw_to_float(u[e]);
     }
-    const float ls = z < 0.0f ? z - log1pf(expf(z)) : -log1pf(expf(-z));
-    p.dec[idx] = expf(ls * p.inv_tau);
+    p.dec[idx] = lr_decay(z, p.form.decay_kind, p.inv_tau);
     p.qf[idx] = cw_to_float(row[p.q_off + c]) * p.q_scale;
     p.kf[idx] = cw_to_float(row[p.k_off + c]);
   }
@@ -330,6 +372,19 @@ __global__ __launch_bounds__(256) void lrs_walk_kernel(SegParams p) {
     const float* q = Qt + t * D;
     const float vv = cw_to_float(proj[row * p.stride + p.v_off + h * V + vc]);
     float o0 = 0.0f, o1 = 0.0f, o2 = 0.0f, o3 = 0.0f;
+    if (MODE == 1 && p.form.bonus) {
+      // the output reads the state before the token joins it, and the token through the bonus
+      const float* bn = p.form.bonus + h * D;
+#pragma unroll
+      for (int d = 0; d < DIM; d += 4) {
+        if (d < D) {
+          o0 += q[d] * (S[d] + bn[d] * k[d] * vv);
+          o1 += q[d + 1] * (S[d + 1] + bn[d + 1] * k[d + 1] * vv);
+          o2 += q[d + 2] * (S[d + 2] + bn[d + 2] * k[d + 2] * vv);
+          o3 += q[d + 3] * (S[d + 3] + bn[d + 3] * k[d + 3] * vv);
+        }
+      }
+    }
 #pragma unroll
     for (int d = 0; d < DIM; d += 4) {
       if (d < D) {  // D is a multiple of 4 here (the host sees to it)
@@ -337,12 +392,12 @@ __global__ __launch_bounds__(256) void lrs_walk_kernel(SegParams p) {
         S[d + 1] = a[d + 1] * S[d + 1] + k[d + 1] * vv;
         S[d + 2] = a[d + 2] * S[d + 2] + k[d + 2] * vv;
         S[d + 3] = a[d + 3] * S[d + 3] + k[d + 3] * vv;
-        if (MODE == 1) {
+        if (MODE == 1 && !p.form.bonus) {
           o0 += q[d] * S[d];
           o1 += q[d + 1] * S[d + 1];
           o2 += q[d + 2] * S[d + 2];
           o3 += q[d + 3] * S[d + 3];
-        } else if (threadIdx.x == 0 && blockIdx.z == 0) {
+        } else if (MODE == 0 && threadIdx.x == 0 && blockIdx.z == 0) {
           A[d] *= a[d]; A[d + 1] *= a[d + 1]; A[d + 2] *= a[d + 2]; A[d + 3] *= a[d + 3];
         }
       }
@@ -373,7 +428,7 @@ __global__ __launch_bounds__(256) void lrs_carry_kernel(SegParams p) {
   const int q_len = p.cu_q[r + 1] - p.cu_q[r];
   if (e >= (int64_t)D * V || slot < 0 || slot >= p.n_slots || q_len <= 0) return;
   const int d = (int)(e / V);
-  float* st = p.state + (((int64_t)slot * p.heads + h) * D) * V + e;
+  float* st = p.state + (int64_t)slot * p.form.state_stride + ((int64_t)h * D) * V + e;
   float S = *st;
   for (int seg = p.req_first[r]; seg < p.req_first[r + 1]; ++seg) {
     if (p.seg_items[4 * seg + 1] >= q_len) break;  // segments past the request's tokens (a batch of fixed shape)
@@ -402,7 +457,7 @@ __global__ __launch_bounds__(256) void lrs_finish_kernel(SegParams p) {
   T* out = (T*)p.out;
   for (int c = lane; c < V; c += 64) {
     float val = o[c] * inv;
-    if (p.norm_w) val *= p.norm_w[c];
+    if (p.norm_w) val *= p.norm_w[h * p.form.norm_w_stride + c];
     if (p.g_off >= 0) {
       const float g = cw_to_float(proj[t * p.stride + p.g_off + h * V + c]);
       val *= g / (1.0f + expf(-g));
@@ -427,13 +482,18 @@ CW_EXPORT int cw_linear_recurrence_segments(int dtype, const void* proj, int64_t
                                             float* state, int n_slots, const int* state_slots, const int* cu_q,
                                             const int* seg_items, int n_segments, int seg_tokens, const int* req_first, float* workspace,
                                             void* out, int n_requests, int n_tokens, int heads, int dim, int vdim, int rank,
-                                            float q_scale, float inv_tau, float eps, hipStream_t stream) {
+                                            float q_scale, float inv_tau, float eps, int decay_kind, const float* bonus,
+                                            int norm_w_stride, const void* u, int64_t u_stride, int64_t state_stride,
+                                            hipStream_t stream) {
   if (n_requests < 0 || n_tokens < 0 || n_segments < 0 || !proj || !a2 || !state || !state_slots || !cu_q || !seg_items ||
       !req_first || !workspace || !out)
     return CW_ERR_ARG;
-  if (heads <= 0 || rank <= 0 || n_slots <= 0 || q_off < 0 || k_off < 0 || v_off < 0 || u_off < 0) return CW_ERR_ARG;
-  if (q_off + heads * dim > stride || k_off + heads * dim > stride || v_off + heads * vdim > stride ||
-      u_off + rank > stride || (g_off >= 0 && g_off + heads * vdim > stride))
+  if (heads <= 0 || rank <= 0 || n_slots <= 0 || q_off < 0 || k_off < 0 || v_off < 0 || u_off < 0 || stride <= 0) return CW_ERR_ARG;
+  if (q_off % stride + heads * dim > stride || k_off % stride + heads * dim > stride || v_off % stride + heads * vdim > stride ||
+      (!u && u_off + rank > stride) || (g_off >= 0 && g_off % stride + heads * vdim > stride))
+    return CW_ERR_ARG;
+  if (decay_kind < 0 || decay_kind > 1 || (norm_w_stride != 0 && norm_w_stride != vdim) || (u && u_stride < rank) ||
+      state_stride < (int64_t)heads * dim * vdim || state_stride > 0x7fffffff)
     return CW_ERR_ARG;
   if (!cw_linear_recurrence_segments_supported(dim, vdim)) return CW_ERR_SIZE;
   if (heads > 65535 || (vdim + 63) / 64 > 65535) return CW_ERR_SIZE;
@@ -445,6 +505,7 @@ CW_EXPORT int cw_linear_recurrence_segments(int dtype, const void* proj, int64_t
   p.seg_items = seg_items; p.req_first = req_first; p.out = out;
   p.heads = heads; p.dim = dim; p.vdim = vdim; p.rank = rank; p.n_slots = n_slots; p.n_tokens = n_tokens;
   p.q_scale = q_scale; p.inv_tau = inv_tau; p.eps = eps;
+  p.form = LinRecForm{decay_kind, bonus, norm_w_stride, u, u_stride, (int)state_stride};
   const int64_t THD = (int64_t)n_tokens * heads * dim;
   p.dec = workspace; p.qf = p.dec + THD; p.kf = p.qf + THD;
   p.added = p.kf + THD;

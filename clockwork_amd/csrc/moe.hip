@@ -3,7 +3,12 @@
 //
 //   1. moe_route:  z = router x in float32, r = 1 / (1 + exp(-z)) (or softmax over the experts),
 //                  the ``top`` largest r, chosen by their z (the lower index first among equals), optionally
-//                  divided by their sum. One workgroup a token.
+//                  divided by their sum. One workgroup a token. Options: a ``correction`` per
+//                  expert joins r for the CHOICE only (the weights stay r); experts in ``groups``
+//                  equal runs of neighbours, a run scored by the sum of its ``group_top`` largest
+//                  choice scores, and only experts of the ``groups_kept`` best runs can be chosen;
+//                  ``extra`` rows behind the router's (gates of the same input) leave their
+//                  logistic values beside the choice.
 //   2. moe_plan:   the (token, choice) pairs sorted by expert into rows; every expert's rows begin
 //                  at a multiple of MOE_TILE_ROWS, so a tile of rows belongs to one expert. One
 //                  workgroup; the tiles' experts and their number stay on the device, and the
@@ -12,7 +17,8 @@
 //   3. moe_up:     per tile, inner = act(gate_e u) * (up_e u) with u = the pair's token row,
 //                  multiplied by its score first when the score weighs the expert's input.
 //   4. moe_down:   per tile, y[pair] = down_e inner (times the score when it weighs the output).
-//   5. moe_combine: out[t] = sum over the token's pairs, in the order of the choices, float32.
+//   5. moe_combine: out[t] = sum over the token's pairs, in the order of the choices, float32;
+//                  then, if there is one, the output of an expert that every token uses, times its gate.
 //
 // Steps 3 and 4 have three kernels. Plain arithmetic on the vector units (tiles of 16 rows): any
 // type and size, and what float32 always runs. For bfloat16 with K a multiple of 8, on the matrix
@@ -37,18 +43,28 @@ typedef __attribute__((ext_vector_type(4))) unsigned int u32x4_t;
 #define MOE_ROUTER_SOFTMAX 1
 
 // ---------------------------------------------------------------- 1. router and choice
+#define MOE_MAX_EXTRA 8
+#define MOE_MAX_GROUP_TOP 64
+struct MoeRouteOptions {
+  const float* correction;  // [E] or null
+  int groups, groups_kept, group_top;   // groups <= 1: every expert can be chosen
+  int extra;                // rows behind the router's E
+  float* extra_out;         // [T, extra]
+};
+
 template <typename T>
 __global__ __launch_bounds__(256) void moe_route_kernel(const T* __restrict__ x, const T* __restrict__ router, int H, int E,
                                                         int top, int kind, int* __restrict__ choice,
-                                                        float* __restrict__ score) {
-  __shared__ float r[MOE_MAX_EXPERTS];  // logits, then scores
-  __shared__ float z[MOE_MAX_EXPERTS];  // logits
+                                                        float* __restrict__ score, MoeRouteOptions opt) {
+  __shared__ float r[MOE_MAX_EXPERTS + MOE_MAX_EXTRA];  // logits, then scores
+  __shared__ float z[MOE_MAX_EXPERTS];  // what the choice compares
+  __shared__ float run_score[MOE_MAX_EXPERTS];
   const int64_t t = blockIdx.x;
   const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
   const T* xr = x + t * H;
   constexpr int V = 16 / (int)sizeof(T);
   const bool vec_ok = H % V == 0 && !((uintptr_t)x & 15) && !((uintptr_t)router & 15);
-  for (int e = wave; e < E; e += 4) {
+  for (int e = wave; e < E + opt.extra; e += 4) {
     const T* w = router + (int64_t)e * H;
     float s = 0.0f;
     if (vec_ok) {  // 16 bytes of each row a lane and step; the order of a lane's sums depends on H alone
@@ -90,6 +106,52 @@ __global__ __launch_bounds__(256) void moe_route_kernel(const T* __restrict__ x,
   } else {
     for (int e = lane; e < E; e += 64) r[e] = 1.0f / (1.0f + expf(-r[e]));
   }
+  for (int x = lane; x < opt.extra; x += 64) opt.extra_out[t * opt.extra + x] = 1.0f / (1.0f + expf(-r[E + x]));
+  if (opt.correction || opt.groups > 1) {
+    // the choice is made on score + correction (which the logits no longer order), and runs are
+    // compared by sums of scores
+    for (int e = lane; e < E; e += 64) z[e] = r[e] + (opt.correction ? opt.correction[e] : 0.0f);
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront", "local");
+    __builtin_amdgcn_wave_barrier();
+    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront", "local");
+  }
+  if (opt.groups > 1) {
+    const int per = E / opt.groups;
+    for (int g = lane; g < opt.groups; g += 64) {
+      // the sum of the run's largest choice scores, taken one after the other: the next one is
+      // the largest that comes after the last in the order (score falling, index rising)
+      float sum = 0.0f, prev = 3.4e38f;
+      int prev_at = -1;
+      for (int n = 0; n < opt.group_top && n < per; ++n) {
+        float best = -3.4e38f;
+        int at = -1;
+        for (int e = g * per; e < (g + 1) * per; ++e) {
+          const float c = z[e];
+          const bool after = c < prev || (c == prev && e > prev_at);
+          if (after && (at < 0 || c > best)) { best = c; at = e; }
+        }
+        if (at < 0) break;
+        sum += best;
+        prev = best;
+        prev_at = at;
+      }
+      run_score[g] = sum;
+    }
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront", "local");
+    __builtin_amdgcn_wave_barrier();
+    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront", "local");
+    // a run is kept if fewer than ``groups_kept`` runs come before it (a larger score, or an equal one and a lower index)
+    for (int e = lane; e < E; e += 64) {
+      const int g = e / per;
+      int ahead = 0;
+      for (int o = 0; o < opt.groups; ++o)
+        ahead += (run_score[o] > run_score[g] || (run_score[o] == run_score[g] && o < g)) ? 1 : 0;
+      if (ahead >= opt.groups_kept) z[e] = -3.4e38f;
+    }
+  }
+  __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront", "local");
+  __builtin_amdgcn_wave_barrier();
+  __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront", "local");
   for (int k = 0; k < top; ++k) {
     // the largest logit still there; among equals the lowest index
     float best = -3.4e38f;
@@ -113,10 +175,11 @@ __global__ __launch_bounds__(256) void moe_route_kernel(const T* __restrict__ x,
 }
 
 // the chosen scores of a token divided by their sum
-__global__ __launch_bounds__(64) void moe_renorm_kernel(float* __restrict__ score, int top) {
+__global__ __launch_bounds__(64) void moe_renorm_kernel(float* __restrict__ score, int top, float eps) {
   const int64_t t = blockIdx.x;
   float sum = 0.0f;
   for (int k = 0; k < top; ++k) sum += score[t * top + k];
+  sum += eps;
   __syncthreads();
   for (int k = threadIdx.x; k < top; k += 64) score[t * top + k] /= sum;
 }
@@ -556,12 +619,15 @@ __global__ __launch_bounds__(256) void moe_gather_bf16_kernel(const bf16_t* __re
 
 // ---------------------------------------------------------------- 5. a token's pairs, added in their order
 template <typename T>
-__global__ void moe_combine_kernel(const T* __restrict__ y, T* __restrict__ out, int top, int H, int64_t total) {
+__global__ void moe_combine_kernel(const T* __restrict__ y, T* __restrict__ out, int top, int H, int64_t total,
+                                   const T* __restrict__ always, const float* __restrict__ always_gate, int gate_stride) {
   for (int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; i < total; i += (int64_t)gridDim.x * blockDim.x) {
     const int64_t t = i / H;
     const int j = (int)(i % H);
     float s = 0.0f;
     for (int k = 0; k < top; ++k) s += cw_to_float(y[(t * top + k) * H + j]);
+    // an expert that every token uses joins last, times its gate if it has one
+    if (always) s += cw_to_float(always[i]) * (always_gate ? always_gate[t * gate_stride] : 1.0f);
     out[i] = cw_from_float<T>(s);
   }
 }
@@ -579,19 +645,25 @@ CW_EXPORT int cw_moe_max_tiles(int n_pairs, int E, int tile_rows) {
 }
 
 CW_EXPORT int cw_moe_route(const void* x, const void* router, int dtype, int T, int H, int E, int top, int kind, int renorm,
-                           int* choice, float* score, hipStream_t stream) {
+                           int* choice, float* score, const float* correction, int groups, int groups_kept, int group_top,
+                           int extra, float* extra_out, float renorm_eps, hipStream_t stream) {
   if (T < 0 || H <= 0 || E <= 0 || top <= 0 || top > E || !x || !router || !choice || !score) return CW_ERR_ARG;
+  if (extra < 0 || extra > MOE_MAX_EXTRA || (extra > 0 && !extra_out)) return CW_ERR_ARG;
+  if (groups > 1 && (E % groups || groups_kept < 1 || groups_kept > groups || group_top < 1 || group_top > MOE_MAX_GROUP_TOP ||
+                     (E / groups) * groups_kept < top))
+    return CW_ERR_ARG;
+  const MoeRouteOptions opt = {correction, groups, groups_kept, group_top, extra, extra_out};
   if (kind != MOE_ROUTER_SIGMOID && kind != MOE_ROUTER_SOFTMAX) return CW_ERR_ARG;
   if (E > MOE_MAX_EXPERTS) return CW_ERR_SIZE;
   if (T == 0) return CW_OK;
   if (dtype == CW_F32)
     hipLaunchKernelGGL(moe_route_kernel<float>, dim3(T), dim3(256), 0, stream, (const float*)x, (const float*)router, H, E, top,
-                       kind, choice, score);
+                       kind, choice, score, opt);
   else if (dtype == CW_BF16)
     hipLaunchKernelGGL(moe_route_kernel<bf16_t>, dim3(T), dim3(256), 0, stream, (const bf16_t*)x, (const bf16_t*)router, H, E,
-                       top, kind, choice, score);
+                       top, kind, choice, score, opt);
   else return CW_ERR_DTYPE;
-  if (renorm) hipLaunchKernelGGL(moe_renorm_kernel, dim3(T), dim3(64), 0, stream, score, top);
+  if (renorm) hipLaunchKernelGGL(moe_renorm_kernel, dim3(T), dim3(64), 0, stream, score, top, renorm_eps);
   return cw_launch_status();
 }
 
@@ -679,16 +751,19 @@ CW_EXPORT int cw_moe_gather(const void* x, void* rows, int dtype, const int* row
   return cw_launch_status();
 }
 
-CW_EXPORT int cw_moe_combine(const void* y, void* out, int dtype, int T, int top, int H, hipStream_t stream) {
-  if (T < 0 || top <= 0 || H <= 0 || !y || !out) return CW_ERR_ARG;
+CW_EXPORT int cw_moe_combine(const void* y, void* out, int dtype, int T, int top, int H, const void* always,
+                             const float* always_gate, int gate_stride, hipStream_t stream) {
+  if (T < 0 || top <= 0 || H <= 0 || !y || !out || (always_gate && (!always || gate_stride < 1))) return CW_ERR_ARG;
   if (T == 0) return CW_OK;
   const int64_t total = (int64_t)T * H;
   int64_t blocks = (total + 255) / 256;
   if (blocks > 262144) blocks = 262144;
   dim3 grid((unsigned)blocks), block(256);
-  if (dtype == CW_F32) hipLaunchKernelGGL(moe_combine_kernel<float>, grid, block, 0, stream, (const float*)y, (float*)out, top, H, total);
+  if (dtype == CW_F32) hipLaunchKernelGGL(moe_combine_kernel<float>, grid, block, 0, stream, (const float*)y, (float*)out, top, H, total,
+                                           (const float*)always, always_gate, gate_stride);
   else if (dtype == CW_BF16)
-    hipLaunchKernelGGL(moe_combine_kernel<bf16_t>, grid, block, 0, stream, (const bf16_t*)y, (bf16_t*)out, top, H, total);
+    hipLaunchKernelGGL(moe_combine_kernel<bf16_t>, grid, block, 0, stream, (const bf16_t*)y, (bf16_t*)out, top, H, total,
+                       (const bf16_t*)always, always_gate, gate_stride);
   else return CW_ERR_DTYPE;
   return cw_launch_status();
 }

@@ -9,7 +9,9 @@
 //             as key and as value); then there is one plane and M = 1.
 //   * mask:   causal; a window of W positions (a token sees itself and the W - 1 before it); or
 //             segments of C positions counted from position 0 (a token sees the earlier tokens of
-//             its own segment).
+//             its own segment). With a window, the first ``keep_first`` positions of a request
+//             stay visible to every later token, at their true positions.
+//   * cap:    scores are squashed before the softmax: cap * tanh(scale * q . k / cap).
 //   * sink:   exp(sink[head]) joins the softmax denominator (no key, no value, not scaled).
 //   * norm:   the head's output is divided by its root mean square over vdim (eps inside the
 //             root) and multiplied by a constant.
@@ -47,6 +49,8 @@ struct RowsAttnParams {
   float scale;
   int head_norm;           // 0 / 1
   float norm_eps, post_mult;
+  int keep_first;          // with a window: positions below this one are seen from anywhere later
+  float softcap;           // > 0: score <- softcap * tanh(score / softcap)
 };
 
 __host__ __device__ inline int ra_key_stride(int maps, int dim) { return maps * dim + 1; }
@@ -121,14 +125,19 @@ __global__ __launch_bounds__(256) void rows_attention_kernel(const RowsAttnParam
   const T* vp = (const T*)p.v_plane;
   const int KI = KC >> 4;
 
-  for (int k0 = first; k0 <= last; k0 += KC) {
+  // the kept first positions that lie before the walk's oldest key are a stretch of their own
+  const int kept_end = (p.mask_kind == RA_MASK_WINDOW && p.keep_first > 0) ? min(p.keep_first, first) : 0;
+  const float inv_cap = p.softcap > 0.0f ? 1.0f / p.softcap : 0.0f;
+  for (int stretch = kept_end > 0 ? 0 : 1; stretch < 2; ++stretch) {
+  const int begin = stretch == 0 ? 0 : first, end = stretch == 0 ? kept_end - 1 : last;
+  for (int k0 = begin; k0 <= end; k0 += KC) {
     __syncthreads();  // the tile of the round before has been read (and the queries are written)
     const int width = M * D;
     for (int i = tid; i < KC * width; i += 256) {
       const int j = i / width, d = i % width;
       const int key = k0 + j;
       float v = 0.0f;
-      if (key <= last) {
+      if (key <= end) {
         const int page = table[key / p.block_size];
         const int64_t slot = (int64_t)page * p.block_size + key % p.block_size;
         if (page >= 0 && slot < p.cache_rows) v = cw_to_float(kp[slot * p.k_row + (int64_t)g * width + d]);
@@ -140,7 +149,7 @@ __global__ __launch_bounds__(256) void rows_attention_kernel(const RowsAttnParam
         const int j = i / V, c = i % V;
         const int key = k0 + j;
         float v = 0.0f;
-        if (key <= last) {
+        if (key <= end) {
           const int page = table[key / p.block_size];
           const int64_t slot = (int64_t)page * p.block_size + key % p.block_size;
           if (page >= 0 && slot < p.cache_rows) v = cw_to_float(vp[slot * p.v_row + (int64_t)g * V + c]);
@@ -162,8 +171,9 @@ __global__ __launch_bounds__(256) void rows_attention_kernel(const RowsAttnParam
         const float* krow = ks + j * kstride + m * D;
         float dot = 0.0f;
         for (int d = 0; d < D; ++d) dot += qrow[d] * krow[d];
-        if (live && key >= lo && key <= pos) {
+        if (live && key <= min(pos, end) && (key >= lo || key < p.keep_first)) {
           s[i] = dot * p.scale;
+          if (p.softcap > 0.0f) s[i] = p.softcap * tanhf(s[i] * inv_cap);
           tile_max = fmaxf(tile_max, s[i]);
         }
       }
@@ -196,6 +206,7 @@ __global__ __launch_bounds__(256) void rows_attention_kernel(const RowsAttnParam
         acc[i] = a;
       }
     }
+  }
   }
   // a row that saw no key and has no sink cannot happen: every token sees itself
   const float inv = run_sum > 0.0f ? 1.0f / run_sum : 0.0f;
@@ -259,12 +270,13 @@ CW_EXPORT int cw_rows_attention(int dtype, const void* q, int64_t q_stride, int6
                                 const int* items, int n_items, const float* sink, const float* lambda, int heads,
                                 int kv_heads, int dim, int vdim, int maps, int block_size, int mask_kind,
                                 int mask_size, float scale, int head_norm, float norm_eps, float post_mult,
-                                hipStream_t stream) {
+                                int keep_first, float softcap, hipStream_t stream) {
   if (n_items < 0 || !q || !out || !k_plane || !v_plane || !block_tables || !ctx_lens || !cu_q || !items)
     return CW_ERR_ARG;
   if (block_size <= 0 || table_width <= 0 || mask_kind < 0 || mask_kind > 2 || (mask_kind != 0 && mask_size < 1))
     return CW_ERR_ARG;
   if (maps == 2 && !lambda) return CW_ERR_ARG;
+  if (keep_first < 0 || (keep_first > 0 && mask_kind != RA_MASK_WINDOW) || softcap < 0.0f) return CW_ERR_ARG;
   const int alias = v_plane == k_plane;
   const int kc = cw_rows_attention_key_chunk(maps, dim, vdim, alias);
   const int hc = cw_rows_attention_heads_per_group(heads, kv_heads, maps);
@@ -280,6 +292,7 @@ CW_EXPORT int cw_rows_attention(int dtype, const void* q, int64_t q_stride, int6
   p.kv_heads = kv_heads; p.dim = dim; p.vdim = vdim; p.maps = maps; p.heads_per_group = hc;
   p.tokens_per_item = RA_ROWS / (hc * maps); p.key_chunk = kc; p.block_size = block_size; p.mask_kind = mask_kind;
   p.mask_size = mask_size; p.scale = scale; p.head_norm = head_norm; p.norm_eps = norm_eps; p.post_mult = post_mult;
+  p.keep_first = keep_first; p.softcap = softcap;
   const size_t smem = ra_lds_floats(maps, dim, vdim, kc, alias) * sizeof(float);
   const int group = heads / kv_heads;
   dim3 grid(n_items, kv_heads, (group + hc - 1) / hc), block(256);
@@ -759,7 +772,7 @@ CW_EXPORT int cw_rows_attention_mfma(const void* q, int64_t q_stride, int64_t q_
   p.ctx_lens = ctx_lens; p.cu_q = cu_q; p.items = items; p.sink = sink; p.lambda = lambda; p.heads = heads;
   p.kv_heads = kv_heads; p.dim = dim; p.vdim = vdim; p.maps = maps; p.heads_per_group = 0; p.tokens_per_item = 16;
   p.key_chunk = RM_KT; p.block_size = block_size; p.mask_kind = mask_kind; p.mask_size = mask_size; p.scale = scale;
-  p.head_norm = head_norm; p.norm_eps = norm_eps; p.post_mult = post_mult;
+  p.head_norm = head_norm; p.norm_eps = norm_eps; p.post_mult = post_mult; p.keep_first = 0; p.softcap = 0.0f;
   RowsMfmaExtra x;
   x.workspace = workspace; x.v_splits = vsp; x.heads_per_wg = maps == 2 ? 4 : 4 * upw;
   const int group = heads / kv_heads;

@@ -470,30 +470,31 @@ CW_EXPORT int cw_gelu_erf(void* x, int dtype, int64_t n, hipStream_t stream) {
 }
 
 // ---------------------------------------------------------------- a * sigmoid(z), in place on a
-// a[t, j] <- a[t, j] / (1 + exp(-z[t, z_off + j])), j < n; z rows are z_stride elements apart.
+// a[t, j] <- a[t, j] / (1 + exp(-z[t, z_off + j / group])), j < n; z rows are z_stride elements
+// apart. group 1: a gate an element; group g: one gate for every run of g elements (a head).
 template <typename T>
 __global__ void sigmoid_mul_kernel(T* __restrict__ a, const T* __restrict__ z, int64_t z_stride, int z_off, int n,
-                                   int64_t total) {
+                                   int group, int64_t total) {
   for (int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; i < total; i += (int64_t)gridDim.x * blockDim.x) {
     const int64_t t = i / n;
-    const int j = (int)(i % n);
+    const int j = (int)(i % n) / group;
     const float g = 1.0f / (1.0f + expf(-cw_to_float(z[t * z_stride + z_off + j])));
     a[i] = cw_from_float<T>(cw_to_float(a[i]) * g);
   }
 }
 
-CW_EXPORT int cw_sigmoid_mul(void* a, const void* z, int dtype, int64_t z_stride, int z_off, int T, int n,
+CW_EXPORT int cw_sigmoid_mul(void* a, const void* z, int dtype, int64_t z_stride, int z_off, int T, int n, int group,
                              hipStream_t stream) {
-  if (T < 0 || n <= 0 || z_off < 0 || z_off + n > z_stride) return CW_ERR_ARG;
+  if (T < 0 || n <= 0 || group <= 0 || n % group || z_off < 0 || z_off + n / group > z_stride) return CW_ERR_ARG;
   if (T == 0) return CW_OK;
   const int64_t total = (int64_t)T * n;
   int64_t blocks = (total + 255) / 256;
   if (blocks > 262144) blocks = 262144;
   dim3 grid((unsigned)blocks), block(256);
   if (dtype == CW_F32)
-    hipLaunchKernelGGL(sigmoid_mul_kernel<float>, grid, block, 0, stream, (float*)a, (const float*)z, z_stride, z_off, n, total);
+    hipLaunchKernelGGL(sigmoid_mul_kernel<float>, grid, block, 0, stream, (float*)a, (const float*)z, z_stride, z_off, n, group, total);
   else if (dtype == CW_BF16)
-    hipLaunchKernelGGL(sigmoid_mul_kernel<bf16_t>, grid, block, 0, stream, (bf16_t*)a, (const bf16_t*)z, z_stride, z_off, n, total);
+    hipLaunchKernelGGL(sigmoid_mul_kernel<bf16_t>, grid, block, 0, stream, (bf16_t*)a, (const bf16_t*)z, z_stride, z_off, n, group, total);
   else return CW_ERR_DTYPE;
   return cw_launch_status();
 }
@@ -748,13 +749,26 @@ CW_EXPORT int cw_stream_norm(const float* resid, const void* w, int w_dtype, flo
 // Values go to v_plane[slot, nv]: the biased value projection, or with v_from_keys the biased key
 // projection as it was before norm and rotation (nv == nkv * dim). A negative slot writes no
 // cache row. One workgroup a token, one wave a vector at a time; float32 inside.
+//
+// Options (HeadNormOptions): ``pairing`` 1 rotates neighbours, (2i, 2i + 1) by freq[i], instead of
+// halves. ``norm`` 0: no norm; 1: norm (and weight), then rotation; 2: rotation, then the rotated
+// vector is divided by ITS root mean square (and multiplied by the weight). The weights may be
+// absent with either norm. ``q_temp_every`` n > 0: every query is multiplied, last, by
+// 1 + q_temp_coef * ln(floor((position + 1) / n) + 1).
 #define HN_MAX_DIM 1024
+struct HeadNormOptions {
+  int pairing, norm, q_temp_every;
+  float q_temp_coef;
+};
+__device__ __forceinline__ float hn_query_factor(const HeadNormOptions& o, int position) {
+  return o.q_temp_every > 0 ? 1.0f + o.q_temp_coef * logf((float)((position + 1) / o.q_temp_every + 1)) : 1.0f;
+}
 template <typename T, typename WT, typename BT>
 __global__ __launch_bounds__(1024) void headnorm_rope_store_kernel(
     T* __restrict__ proj, int64_t stride, int q_off, int k_off, int v_off, int nqv, int nkv, int dim, int nv,
     const BT* __restrict__ bias, const WT* __restrict__ qw, const WT* __restrict__ kw, float eps,
     const int* __restrict__ positions, const float* __restrict__ freq, int rdims, const int* __restrict__ slots,
-    T* __restrict__ k_plane, T* __restrict__ v_plane, int v_from_keys, int64_t cache_rows) {
+    T* __restrict__ k_plane, T* __restrict__ v_plane, int v_from_keys, int64_t cache_rows, HeadNormOptions opt) {
   extern __shared__ float hn_vals[];  // [waves][dim], then the token's cosines and sines [2][rdims / 2]
   const int64_t t = blockIdx.x;
   T* row = proj + t * stride;
@@ -775,6 +789,7 @@ __global__ __launch_bounds__(1024) void headnorm_rope_store_kernel(
   float* sines = cosines + half;
   for (int i = threadIdx.x; i < half; i += blockDim.x) sincosf(pos * freq[i], &sines[i], &cosines[i]);
   __syncthreads();
+  const float q_factor = hn_query_factor(opt, positions ? positions[t] : 0);
   for (int vec = wave; vec < nqv + nkv; vec += n_waves) {
     const bool is_q = vec < nqv;
     if (!is_q && slot < 0) continue;
@@ -786,23 +801,32 @@ __global__ __launch_bounds__(1024) void headnorm_rope_store_kernel(
       vals[j] = v;
       ss += v * v;
     }
-    const float inv = w ? 1.0f / sqrtf(cw_wave_sum(ss) / (float)dim + eps) : 1.0f;
+    const float inv = opt.norm == 1 ? 1.0f / sqrtf(cw_wave_sum(ss) / (float)dim + eps) : 1.0f;
     __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront", "local");
     __builtin_amdgcn_wave_barrier();
     __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront", "local");
+    // element j after the norm that comes first (if that is the order) and the rotation
+    auto turned = [&](int j) -> float {
+      const bool pre = opt.norm == 1;
+      if (j >= rdims) return vals[j] * (pre ? inv * (w ? cw_to_float(w[j]) : 1.0f) : 1.0f);
+      const int i = opt.pairing ? j >> 1 : (j < half ? j : j - half);
+      const int ja = opt.pairing ? 2 * i : i, jb = opt.pairing ? 2 * i + 1 : i + half;
+      const float a = vals[ja] * (pre ? inv * (w ? cw_to_float(w[ja]) : 1.0f) : 1.0f);
+      const float b = vals[jb] * (pre ? inv * (w ? cw_to_float(w[jb]) : 1.0f) : 1.0f);
+      const float s = sines[i], c = cosines[i];
+      return j == ja ? a * c - b * s : b * c + a * s;
+    };
+    float inv_after = 1.0f;
+    if (opt.norm == 2) {
+      float s2 = 0.0f;
+      for (int j = lane; j < dim; j += 64) { const float r = turned(j); s2 += r * r; }
+      inv_after = 1.0f / sqrtf(cw_wave_sum(s2) / (float)dim + eps);
+    }
     T* dst = is_q ? row + base : k_plane + slot * ((int64_t)nkv * dim) + (int64_t)(vec - nqv) * dim;
     for (int j = lane; j < dim; j += 64) {
-      float v;
-      if (j < rdims) {
-        const int i = j < half ? j : j - half;
-        const float a = vals[i] * inv * (w ? cw_to_float(w[i]) : 1.0f);
-        const float b = vals[i + half] * inv * (w ? cw_to_float(w[i + half]) : 1.0f);
-        const float s = sines[i], c = cosines[i];
-        v = j < half ? a * c - b * s : b * c + a * s;
-      } else {
-        v = vals[j] * inv * (w ? cw_to_float(w[j]) : 1.0f);
-      }
-      dst[j] = cw_from_float<T>(v);
+      float v = turned(j);
+      if (opt.norm == 2) v *= inv_after * (w ? cw_to_float(w[j]) : 1.0f);
+      dst[j] = cw_from_float<T>(is_q ? v * q_factor : v);
     }
     __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront", "local");
     __builtin_amdgcn_wave_barrier();
@@ -821,7 +845,7 @@ __global__ __launch_bounds__(256) void headnorm_rope_store_vec_kernel(
     bf16_t* __restrict__ proj, int64_t stride, int q_off, int k_off, int v_off, int nqv, int nkv, int dim, int nv,
     const BT* __restrict__ bias, const WT* __restrict__ qw, const WT* __restrict__ kw, float eps,
     const int* __restrict__ positions, const float* __restrict__ freq, int rdims, const int* __restrict__ slots,
-    bf16_t* __restrict__ k_plane, bf16_t* __restrict__ v_plane, int v_from_keys, int64_t cache_rows) {
+    bf16_t* __restrict__ k_plane, bf16_t* __restrict__ v_plane, int v_from_keys, int64_t cache_rows, HeadNormOptions opt) {
   extern __shared__ float hn_vals[];  // the token's cosines and sines [2][rdims / 2]
   const int64_t t = blockIdx.x;
   bf16_t* row = proj + t * stride;
@@ -842,9 +866,12 @@ __global__ __launch_bounds__(256) void headnorm_rope_store_vec_kernel(
   __syncthreads();
   const int lanes = dim >> 3, per_wave = 64 / lanes;   // lanes of a vector (a power of two), vectors of a wave
   const int sub = lane & (lanes - 1), j0 = sub * 8;
+  // halves: a rotated element's partner lies dims / 2 elements away, in another lane; neighbours:
+  // both elements of a pair lie in the lane itself
   const bool rotated = j0 < rdims, low = j0 < half;
-  const int partner = rotated ? (low ? lane + (half >> 3) : lane - (half >> 3)) : lane;
+  const int partner = (rotated && !opt.pairing) ? (low ? lane + (half >> 3) : lane - (half >> 3)) : lane;
   const int n_vec = nqv + nkv;
+  const float q_factor = hn_query_factor(opt, positions ? positions[t] : 0);
   for (int first = 0; first < n_vec; first += 4 * per_wave) {  // every lane of a wave stays for the exchanges
     const int vec = first + wave * per_wave + lane / lanes;
     const bool is_q = vec < nqv;
@@ -870,26 +897,40 @@ __global__ __launch_bounds__(256) void headnorm_rope_store_vec_kernel(
 #pragma unroll
     for (int i = 0; i < 8; ++i) ss += v[i] * v[i];
     for (int off = 1; off < lanes; off <<= 1) ss += __shfl_xor(ss, off, 64);
-    const float inv = w ? 1.0f / sqrtf(ss / (float)dim + eps) : 1.0f;
+    const bool pre = opt.norm == 1;
+    const float inv = pre ? 1.0f / sqrtf(ss / (float)dim + eps) : 1.0f;
     float pv[8];
 #pragma unroll
-    for (int i = 0; i < 8; ++i) pv[i] = __shfl(v[i], partner, 64);
+    for (int i = 0; i < 8; ++i) pv[i] = opt.pairing ? v[i ^ 1] : __shfl(v[i], partner, 64);
+    float r[8];
+#pragma unroll
+    for (int i = 0; i < 8; ++i) {
+      if (rotated) {
+        // ja, jb: the pair's two elements; ``mine_first``: this element is the pair's first
+        const bool mine_first = opt.pairing ? !(i & 1) : low;
+        const int idx = opt.pairing ? (j0 + i) >> 1 : (low ? j0 : j0 - half) + i;
+        const int ja = opt.pairing ? 2 * idx : idx, jb = opt.pairing ? 2 * idx + 1 : idx + half;
+        const float a = (mine_first ? v[i] : pv[i]) * (pre ? inv * (w ? cw_to_float(w[ja]) : 1.0f) : 1.0f);
+        const float b = (mine_first ? pv[i] : v[i]) * (pre ? inv * (w ? cw_to_float(w[jb]) : 1.0f) : 1.0f);
+        const float sn = live ? sines[idx] : 0.0f, c = live ? cosines[idx] : 0.0f;
+        r[i] = mine_first ? a * c - b * sn : b * c + a * sn;
+      } else {
+        r[i] = v[i] * (pre ? inv * (w ? cw_to_float(w[j0 + i]) : 1.0f) : 1.0f);
+      }
+    }
+    if (opt.norm == 2) {
+      float s2 = 0.0f;
+#pragma unroll
+      for (int i = 0; i < 8; ++i) s2 += r[i] * r[i];
+      for (int off = 1; off < lanes; off <<= 1) s2 += __shfl_xor(s2, off, 64);
+      const float inv_after = 1.0f / sqrtf(s2 / (float)dim + eps);
+#pragma unroll
+      for (int i = 0; i < 8; ++i) r[i] *= inv_after * (w ? cw_to_float(w[j0 + i]) : 1.0f);
+    }
     if (!live) continue;
     uint16_t o[8];
 #pragma unroll
-    for (int i = 0; i < 8; ++i) {
-      float r;
-      if (rotated) {
-        const int idx = (low ? j0 : j0 - half) + i;
-        const float a = (low ? v[i] : pv[i]) * inv * (w ? cw_to_float(w[idx]) : 1.0f);
-        const float b = (low ? pv[i] : v[i]) * inv * (w ? cw_to_float(w[idx + half]) : 1.0f);
-        const float sn = sines[idx], c = cosines[idx];
-        r = low ? a * c - b * sn : b * c + a * sn;
-      } else {
-        r = v[i] * inv * (w ? cw_to_float(w[j0 + i]) : 1.0f);
-      }
-      o[i] = cw_float_to_bf16_bits(r);
-    }
+    for (int i = 0; i < 8; ++i) o[i] = cw_float_to_bf16_bits(is_q ? r[i] * q_factor : r[i]);
     cw_u32x4_t packed;
 #pragma unroll
     for (int i = 0; i < 4; ++i) packed[i] = (uint32_t)o[2 * i] | ((uint32_t)o[2 * i + 1] << 16);
@@ -902,8 +943,11 @@ CW_EXPORT int cw_headnorm_rope_store(void* proj, int dtype, int64_t stride, int 
                                      int dim, int nv, const void* bias, int b_dtype, const void* qw, const void* kw,
                                      int w_dtype, float eps, const int* positions, const float* freq, int rdims,
                                      const int* slots, void* k_plane, void* v_plane, int v_from_keys, int64_t cache_rows,
-                                     int T, hipStream_t stream) {
+                                     int T, int pairing, int norm, float q_temp_coef, int q_temp_every,
+                                     hipStream_t stream) {
   if (T < 0 || nqv < 0 || nkv < 0 || dim <= 0 || nv < 0 || rdims < 0 || rdims > dim || (rdims & 1)) return CW_ERR_ARG;
+  if (pairing < 0 || pairing > 1 || norm < 0 || norm > 2 || q_temp_every < 0 || (q_temp_every > 0 && !positions)) return CW_ERR_ARG;
+  const HeadNormOptions opt = {pairing, norm, q_temp_every, q_temp_coef};
   if (dim > HN_MAX_DIM) return CW_ERR_SIZE;
   if (q_off < 0 || k_off < 0 || v_off < 0 || q_off + (int64_t)nqv * dim > stride || k_off + (int64_t)nkv * dim > stride)
     return CW_ERR_ARG;
@@ -912,13 +956,13 @@ CW_EXPORT int cw_headnorm_rope_store(void* proj, int dtype, int64_t stride, int 
   if ((qw == nullptr) != (kw == nullptr)) return CW_ERR_ARG;
   if (T == 0) return CW_OK;
   // bfloat16 vectors that lanes of 8 elements tile: the kernel of 16-byte accesses
-  if (dtype == CW_BF16 && dim >= 8 && dim <= 512 && !(dim & (dim - 1)) && !(rdims & 15) && !(q_off & 7) && !(k_off & 7) &&
+  if (dtype == CW_BF16 && dim >= 8 && dim <= 512 && !(dim & (dim - 1)) && !(rdims & (pairing ? 7 : 15)) && !(q_off & 7) && !(k_off & 7) &&
       !(stride & 7) && !((uintptr_t)proj & 15) && !((uintptr_t)k_plane & 15)) {
     const size_t lds_vec = (size_t)(rdims ? rdims : 2) * sizeof(float);
 #define CW_LAUNCH_VEC(WT_, BT_)                                                                                         \
   hipLaunchKernelGGL((headnorm_rope_store_vec_kernel<WT_, BT_>), dim3(T), dim3(256), lds_vec, stream, (bf16_t*)proj, stride, \
                      q_off, k_off, v_off, nqv, nkv, dim, nv, (const BT_*)bias, (const WT_*)qw, (const WT_*)kw, eps, positions, \
-                     freq, rdims, slots, (bf16_t*)k_plane, (bf16_t*)v_plane, v_from_keys, cache_rows)
+                     freq, rdims, slots, (bf16_t*)k_plane, (bf16_t*)v_plane, v_from_keys, cache_rows, opt)
     const int wt_v = qw ? w_dtype : CW_BF16, bt_v = bias ? b_dtype : CW_BF16;
     if (wt_v == CW_BF16 && bt_v == CW_BF16) CW_LAUNCH_VEC(bf16_t, bf16_t);
     else if (wt_v == CW_F32 && bt_v == CW_BF16) CW_LAUNCH_VEC(float, bf16_t);
@@ -937,7 +981,7 @@ CW_EXPORT int cw_headnorm_rope_store(void* proj, int dtype, int64_t stride, int 
 #define CW_LAUNCH(T_, WT_, BT_)                                                                                          \
   hipLaunchKernelGGL((headnorm_rope_store_kernel<T_, WT_, BT_>), grid, block, lds, stream, (T_*)proj, stride, q_off, k_off, \
                      v_off, nqv, nkv, dim, nv, (const BT_*)bias, (const WT_*)qw, (const WT_*)kw, eps, positions, freq, rdims, \
-                     slots, (T_*)k_plane, (T_*)v_plane, v_from_keys, cache_rows)
+                     slots, (T_*)k_plane, (T_*)v_plane, v_from_keys, cache_rows, opt)
   const int wt = qw ? w_dtype : dtype, bt = bias ? b_dtype : dtype;
   if (dtype == CW_F32 && wt == CW_F32 && bt == CW_F32) CW_LAUNCH(float, float, float);
   else if (dtype == CW_BF16 && wt == CW_BF16 && bt == CW_BF16) CW_LAUNCH(bf16_t, bf16_t, bf16_t);
@@ -982,5 +1026,99 @@ CW_EXPORT int cw_scale(float* x, int64_t n, float s, hipStream_t stream) {
   int64_t blocks = (n + 255) / 256;
   if (blocks > 262144) blocks = 262144;
   hipLaunchKernelGGL(scale_kernel, dim3((unsigned)blocks), dim3(256), 0, stream, x, n, s);
+  return cw_launch_status();
+}
+
+// ---------------------------------------------------------------- mixes of a token with the one before it
+// out[s][t] = x[t] + (before[t] - x[t]) * mu[s], s < n_mix, float32 inside: ``before`` is the row
+// of the request's token one position earlier: the row above in x, or for the first token of a
+// request's portion what the request's state slot holds at ``prev_off`` (state rows are
+// state_stride floats; a request's first token ever finds zeros there, its slot being fresh).
+// items: (request, first token, tokens, 0), up to SHIFT_TOKENS tokens each. The workgroup of a
+// request's first item then leaves the portion's last row in the slot, for the next step: it alone
+// reads and writes the slot, in that order.
+#define SHIFT_TOKENS 16
+template <typename T, typename WT>
+__global__ __launch_bounds__(256) void shift_mix_kernel(const T* __restrict__ x, const WT* __restrict__ mu, int n_mix,
+                                                        float* __restrict__ state, int64_t state_stride, int64_t prev_off,
+                                                        int n_slots, const int* __restrict__ state_slots,
+                                                        const int* __restrict__ cu_q, const int* __restrict__ items,
+                                                        T* __restrict__ out, int64_t n_tokens, int W) {
+  const int* item = items + 4 * (int64_t)blockIdx.x;
+  const int req = item[0], tok0 = item[1];
+  const int row0 = cu_q[req], q_len = cu_q[req + 1] - row0;
+  if (tok0 >= q_len) return;  // an item past the request's tokens (a batch of fixed shape)
+  const int ntok = min(min(item[2], SHIFT_TOKENS), q_len - tok0);
+  const int slot = state_slots[req];
+  const bool has_slot = slot >= 0 && slot < n_slots;
+  float* kept = has_slot ? state + (int64_t)slot * state_stride + prev_off : nullptr;
+  for (int i = 0; i < ntok; ++i) {
+    const int64_t row = (int64_t)row0 + tok0 + i;
+    const bool first = tok0 + i == 0;
+    for (int j = threadIdx.x; j < W; j += 256) {
+      const float v = cw_to_float(x[row * W + j]);
+      const float b = first ? (kept ? kept[j] : 0.0f) : cw_to_float(x[(row - 1) * W + j]);
+      for (int s = 0; s < n_mix; ++s)
+        out[((int64_t)s * n_tokens + row) * W + j] = cw_from_float<T>(v + (b - v) * cw_to_float(mu[(int64_t)s * W + j]));
+    }
+  }
+  if (tok0 == 0 && kept) {
+    __syncthreads();  // every thread has read what the slot held
+    const int64_t last = (int64_t)row0 + q_len - 1;
+    for (int j = threadIdx.x; j < W; j += 256) kept[j] = cw_to_float(x[last * W + j]);
+  }
+}
+
+CW_EXPORT int cw_shift_mix(const void* x, int dtype, const void* mu, int mu_dtype, int n_mix, float* state,
+                           int64_t state_stride, int64_t prev_off, int n_slots, const int* state_slots, const int* cu_q,
+                           const int* items, int n_items, void* out, int64_t n_tokens, int W, hipStream_t stream) {
+  if (!x || !mu || !state || !state_slots || !cu_q || !items || !out) return CW_ERR_ARG;
+  if (n_mix < 1 || n_items < 0 || n_tokens < 0 || W < 1 || n_slots < 1 || prev_off < 0 || prev_off + W > state_stride)
+    return CW_ERR_ARG;
+  if (n_items == 0 || n_tokens == 0) return CW_OK;
+#define CW_LAUNCH(T_, WT_)                                                                                          \
+  hipLaunchKernelGGL((shift_mix_kernel<T_, WT_>), dim3(n_items), dim3(256), 0, stream, (const T_*)x, (const WT_*)mu, n_mix, \
+                     state, state_stride, prev_off, n_slots, state_slots, cu_q, items, (T_*)out, n_tokens, W)
+  if (dtype == CW_F32 && mu_dtype == CW_F32) CW_LAUNCH(float, float);
+  else if (dtype == CW_BF16 && mu_dtype == CW_BF16) CW_LAUNCH(bf16_t, bf16_t);
+  else if (dtype == CW_BF16 && mu_dtype == CW_F32) CW_LAUNCH(bf16_t, float);
+  else return CW_ERR_DTYPE;
+#undef CW_LAUNCH
+  return cw_launch_status();
+}
+
+// ---------------------------------------------------------------- the stream beside the model's input
+// resid[t] += a[t] + b[t] (what is still pending, either may be absent), then
+// image[t] = [resid[t], input[t], e] in the activation type, e being ``extra`` columns that are 0
+// but for a 1 in column ``hot``: the operand of a product that re-enters the stream from itself
+// and the model's input, and picks one of ``extra`` learned rows on the way. float32 sums.
+template <typename T>
+__global__ __launch_bounds__(256) void stream_beside_input_kernel(float* __restrict__ resid, const T* __restrict__ a,
+                                                                  const T* __restrict__ b, const float* __restrict__ input,
+                                                                  T* __restrict__ image, int H, int extra, int hot) {
+  const int64_t t = blockIdx.x;
+  T* row = image + t * (2 * (int64_t)H + extra);
+  for (int j = threadIdx.x; j < H; j += 256) {
+    float v = resid[t * H + j];
+    if (a) v += cw_to_float(a[t * H + j]);
+    if (b) v += cw_to_float(b[t * H + j]);
+    if (a || b) resid[t * H + j] = v;
+    row[j] = cw_from_float<T>(v);
+    row[H + j] = cw_from_float<T>(input[t * H + j]);
+  }
+  for (int e = threadIdx.x; e < extra; e += 256) row[2 * H + e] = cw_from_float<T>(e == hot ? 1.0f : 0.0f);
+}
+
+CW_EXPORT int cw_stream_beside_input(float* resid, const void* a, const void* b, const float* input, void* image, int dtype,
+                                     int T, int H, int extra, int hot, hipStream_t stream) {
+  if (T < 0 || H <= 0 || extra < 0 || hot < -1 || hot >= (extra ? extra : 1) || !resid || !input || !image) return CW_ERR_ARG;
+  if (T == 0) return CW_OK;
+  if (dtype == CW_F32)
+    hipLaunchKernelGGL(stream_beside_input_kernel<float>, dim3(T), dim3(256), 0, stream, resid, (const float*)a, (const float*)b,
+                       input, (float*)image, H, extra, hot);
+  else if (dtype == CW_BF16)
+    hipLaunchKernelGGL(stream_beside_input_kernel<bf16_t>, dim3(T), dim3(256), 0, stream, resid, (const bf16_t*)a,
+                       (const bf16_t*)b, input, (bf16_t*)image, H, extra, hot);
+  else return CW_ERR_DTYPE;
   return cw_launch_status();
 }

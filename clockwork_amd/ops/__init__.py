@@ -129,24 +129,26 @@ def _declare(name: str, lib: ctypes.CDLL) -> None:
             "cw_qk_rownorm_store": [P, I, L, I, I, I, I, I, I, P, P, I, F, P, P, P, L, I, P],
             "cw_add_dyt": [P, P, I, F, P, P, P, I, P, P, I, P, I, I, P],
             "cw_gelu_erf": [P, I, L, P],
-            "cw_sigmoid_mul": [P, P, I, L, I, I, I, P],
+            "cw_sigmoid_mul": [P, P, I, L, I, I, I, I, P],
             "cw_bias_store": [P, I, L, I, I, I, I, I, I, P, I, P, P, P, L, I, P],
             "cw_latent_store": [P, I, L, I, I, I, I, I, I, P, P, I, F, P, P, P, P, P, L, I, P],
             "cw_rotate_part": [P, I, L, L, I, P, L, L, I, I, I, I, P, P, I, P],
             "cw_branch_norm_add": [P, P, P, I, F, F, F, P, I, I, I, P],
             "cw_stream_norm": [P, P, I, F, F, P, I, P, I, I, P],
-            "cw_headnorm_rope_store": [P, I, L, I, I, I, I, I, I, I, P, I, P, P, I, F, P, P, I, P, P, P, I, L, I, P],
+            "cw_headnorm_rope_store": [P, I, L, I, I, I, I, I, I, I, P, I, P, P, I, F, P, P, I, P, P, P, I, L, I, I, I, F, I, P],
+            "cw_shift_mix": [P, I, P, I, I, P, L, L, I, P, P, P, I, P, L, I, P],
+            "cw_stream_beside_input": [P, P, P, P, P, I, I, I, I, I, P],
             "cw_relu_squared": [P, I, L, P],
             "cw_scale": [P, L, F, P],
         },
         "moe": {
             "cw_moe_tile_rows": [I],
             "cw_moe_max_tiles": [I, I, I],
-            "cw_moe_route": [P, P, I, I, I, I, I, I, I, P, P, P],
+            "cw_moe_route": [P, P, I, I, I, I, I, I, I, P, P, P, I, I, I, I, P, F, P],
             "cw_moe_plan": [P, I, I, I, P, I, P, I, P, P],
             "cw_moe_expert_product": [I, I, P, P, P, I, P, P, P, I, P, I, I, I, I, P],
             "cw_moe_gather": [P, P, I, P, P, I, I, P, I, I, I, P],
-            "cw_moe_combine": [P, P, I, I, I, I, P],
+            "cw_moe_combine": [P, P, I, I, I, I, P, P, I, P],
         },
         "rows_attention": {
             "cw_rows_attention_key_chunk": [I, I, I, I],
@@ -157,7 +159,8 @@ def _declare(name: str, lib: ctypes.CDLL) -> None:
             "cw_rows_mfma_workspace_floats": [I, I, I, I, I, I, I, I],
             "cw_rows_attention_mfma": [P, L, L, P, L, L, P, P, I, I, L, P, I, P, P, P, I, P, P, I, I, I, I, I, I, I, I, F, I, F, F,
                                        I, P, L, P],
-            "cw_rows_attention": [I, P, L, L, P, L, L, P, P, I, I, L, P, I, P, P, P, I, P, P, I, I, I, I, I, I, I, I, F, I, F, F, P],
+            "cw_rows_attention": [I, P, L, L, P, L, L, P, P, I, I, L, P, I, P, P, P, I, P, P, I, I, I, I, I, I, I, I, F, I, F, F,
+                                  I, F, P],
         },
         "sink_attention": {
             "cw_sink_attention_max_bq": [I, I, I, I],
@@ -170,11 +173,11 @@ def _declare(name: str, lib: ctypes.CDLL) -> None:
         },
         "linear_recurrence": {
             "cw_linear_recurrence_supported": [I, I],
-            "cw_linear_recurrence": [I, P, L, I, I, I, I, I, P, P, P, P, I, P, P, P, I, I, I, I, I, F, F, F, P],
+            "cw_linear_recurrence": [I, P, L, I, I, I, I, I, P, P, P, P, I, P, P, P, I, I, I, I, I, F, F, F, I, P, I, P, L, L, P],
             "cw_linear_recurrence_segments_supported": [I, I],
             "cw_linear_recurrence_segments_workspace_floats": [I, I, I, I, I],
             "cw_linear_recurrence_segments": [I, P, L, I, I, I, I, I, P, P, P, P, I, P, P, P, I, I, P, P, P, I, I, I, I, I, I,
-                                              F, F, F, P],
+                                              F, F, F, I, P, I, P, L, L, P],
         },
         "sampling": {
             "cw_argmax_chunks": [I],
@@ -1440,28 +1443,69 @@ def linear_recurrence_supported(dim: int, vdim: int) -> bool:
     return bool(_load("linear_recurrence").cw_linear_recurrence_supported(dim, vdim))
 
 
-def linear_recurrence(proj, q_off: int, k_off: int, v_off: int, g_off: int, u_off: int, a2, a2_bias, norm_weight, state,
-                      state_slots, cu_q, n_requests: int, heads: int, dim: int, vdim: int, q_scale: float, tau: float,
-                      eps: float) -> torch.Tensor:
-    """The decayed recurrence S <- diag(a) S + k v^T, o = S^T (q_scale q) over the step's tokens,
-    request by request from each request's slot of ``state`` (float32 [slots, heads, dim, vdim],
-    updated in place). Rows of ``proj`` hold q, k (heads * dim), v, the output gate (heads * vdim;
-    ``g_off`` < 0: none) and the decay's low-rank input (``a2`` [heads * dim, rank] maps it to
-    z; a = sigmoid(z + bias)^(1/tau)). The outputs are RMS-normed over vdim with ``norm_weight``
-    (None: not) and multiplied by silu(gate). Returns [T, heads * vdim]."""
-    _gpu(proj, a2, a2_bias, norm_weight, state, state_slots, cu_q)
-    T, width = proj.shape
+RECURRENCE_DECAYS = {"sigmoid_power": 0, "double_exp": 1}
+
+
+def _recurrence_operands(proj, q_off, k_off, v_off, g_off, u_off, a2, a2_bias, norm_weight, state, heads, dim, vdim, decay, bonus,
+                         decay_input):
+    """Checks shared by the two recurrence entry points; returns (T, row stride, the five offsets
+    in elements, the trailing arguments of the C call after eps)."""
+    _need(decay in RECURRENCE_DECAYS, f"decay {decay!r}: expected one of {sorted(RECURRENCE_DECAYS)}")
+    if proj.dim() == 3:
+        # planes one behind the other, [planes, T, heads * dim]: an offset names a plane
+        P, T, width = proj.shape
+        _need(proj.is_contiguous() and width == heads * dim and dim == vdim, "planes hold rows of heads * dim (== heads * vdim) elements")
+        _need(decay_input is not None, "with planes the decay input is a tensor of its own")
+        _need(all(0 <= o < P for o in (q_off, k_off, v_off)) and g_off < P, "an offset names a plane")
+        _need(P * T * width < 2 ** 31, "the planes outgrow 32-bit offsets")
+        plane = T * width
+        q_off, k_off, v_off, g_off = q_off * plane, k_off * plane, v_off * plane, (g_off * plane if g_off >= 0 else -1)
+        u_off = 0
+    else:
+        T, width = proj.shape
     _need(a2.dim() == 2 and a2.shape[0] == heads * dim and a2.dtype == proj.dtype, "a2 must be [heads * dim, rank] in the activation type")
     _need(a2_bias is None or (a2_bias.dtype == torch.float32 and a2_bias.numel() == heads * dim), "the decay bias must be float32 [heads * dim]")
-    _need(norm_weight is None or (norm_weight.dtype == torch.float32 and norm_weight.numel() == vdim), "the norm weight must be float32 [vdim]")
-    _need(state.dtype == torch.float32 and tuple(state.shape[1:]) == (heads, dim, vdim), "the state must be float32 [slots, heads, dim, vdim]")
+    _need(norm_weight is None or (norm_weight.dtype == torch.float32 and norm_weight.numel() in (vdim, heads * vdim)),
+          "the norm weight must be float32 [vdim] or [heads * vdim]")
+    _need(bonus is None or (bonus.dtype == torch.float32 and bonus.numel() == heads * dim), "the bonus must be float32 [heads, dim]")
+    _need(state.dtype == torch.float32 and state.dim() >= 2 and state.is_contiguous() and state[0].numel() >= heads * dim * vdim,
+          "the state must be float32 [slots, >= heads * dim * vdim]")
+    u_stride = 0
+    if decay_input is not None:
+        _need(tuple(decay_input.shape) == (T, a2.shape[1]) and decay_input.dtype == proj.dtype and decay_input.is_contiguous(),
+              "the decay input must be [T, rank] in the activation type")
+        u_stride = a2.shape[1]
+    per_head = norm_weight is not None and norm_weight.numel() == heads * vdim and heads > 1
+    tail = (RECURRENCE_DECAYS[decay], _ptr(bonus), vdim if per_head else 0, _ptr(decay_input), u_stride, state[0].numel())
+    return T, width, (int(q_off), int(k_off), int(v_off), int(g_off), int(u_off)), tail
+
+
+def linear_recurrence(proj, q_off: int, k_off: int, v_off: int, g_off: int, u_off: int, a2, a2_bias, norm_weight, state,
+                      state_slots, cu_q, n_requests: int, heads: int, dim: int, vdim: int, q_scale: float, tau: float,
+                      eps: float, decay: str = "sigmoid_power", bonus=None, decay_input=None) -> torch.Tensor:
+    """The decayed recurrence S <- diag(a) S + k v^T, o = S^T (q_scale q) over the step's tokens,
+    request by request from each request's slot of ``state`` (float32 [slots, ...]: a slot's
+    first heads * dim * vdim floats are the matrices, updated in place). Rows of ``proj`` hold q,
+    k (heads * dim), v, the output gate (heads * vdim; ``g_off`` < 0: none) and the decay's
+    low-rank input (``a2`` [heads * dim, rank] maps it to z; a = sigmoid(z + bias)^(1/tau)). The
+    outputs are RMS-normed over vdim with ``norm_weight`` ([vdim] for all heads or [heads * vdim];
+    None: not) and multiplied by silu(gate). Returns [T, heads * vdim].
+
+    ``proj`` [planes, T, heads * dim]: q, k, v and the gate are planes, the offsets their numbers.
+    ``decay_input`` [T, rank]: the decay's input as a tensor of its own. ``decay`` "double_exp":
+    a = exp(-exp(a2 tanh(input) + bias)). ``bonus`` float32 [heads, dim]: the output reads the
+    state before the token joins it and the token itself through the bonus,
+    o = (S + diag(bonus) k v^T)^T q, then S <- diag(a) S + k v^T."""
+    _gpu(proj, a2, a2_bias, norm_weight, state, state_slots, cu_q, bonus, decay_input)
+    T, width, offs, tail = _recurrence_operands(proj, q_off, k_off, v_off, g_off, u_off, a2, a2_bias, norm_weight, state, heads,
+                                                dim, vdim, decay, bonus, decay_input)
     _i32(state_slots, n_requests, "state_slots")
     _i32(cu_q, n_requests + 1, "cu_q")
     out = torch.empty((T, heads * vdim), dtype=proj.dtype, device=proj.device)
     _check(_load("linear_recurrence").cw_linear_recurrence(
-        dtype_code(proj.dtype), _ptr(proj), width, q_off, k_off, v_off, g_off, u_off, _ptr(a2), _ptr(a2_bias),
+        dtype_code(proj.dtype), _ptr(proj), width, *offs, _ptr(a2), _ptr(a2_bias),
         _ptr(norm_weight), _ptr(state), state.shape[0], _ptr(state_slots), _ptr(cu_q), _ptr(out), n_requests, heads, dim,
-        vdim, a2.shape[1], float(q_scale), 1.0 / float(tau), float(eps), _stream()), "linear_recurrence")
+        vdim, a2.shape[1], float(q_scale), 1.0 / float(tau), float(eps), *tail, _stream()), "linear_recurrence")
     return out
 
 
@@ -1472,19 +1516,16 @@ def linear_recurrence_segments_supported(dim: int, vdim: int) -> bool:
 def linear_recurrence_segments(proj, q_off: int, k_off: int, v_off: int, g_off: int, u_off: int, a2, a2_bias, norm_weight,
                                state, state_slots, cu_q, seg_items, n_segments: int, seg_tokens: int, req_first,
                                n_requests: int, heads: int, dim: int, vdim: int, q_scale: float, tau: float,
-                               eps: float) -> torch.Tensor:
+                               eps: float, decay: str = "sigmoid_power", bonus=None, decay_input=None) -> torch.Tensor:
     """``linear_recurrence`` for steps with long portions: the tokens are cut into segments that
     are walked side by side (each from a zero state, then the segments' start states are carried
     from the request's slot, then each is walked again for its outputs). ``seg_items`` int32
     [n_segments, 4]: (request, first token of the segment in the request's portion, tokens, 0),
     a request's segments in order and together, none longer than ``seg_tokens``; ``req_first`` int32 [R + 1]: where each
     request's segments begin. The same arguments and result otherwise."""
-    _gpu(proj, a2, a2_bias, norm_weight, state, state_slots, cu_q, seg_items, req_first)
-    T, width = proj.shape
-    _need(a2.dim() == 2 and a2.shape[0] == heads * dim and a2.dtype == proj.dtype, "a2 must be [heads * dim, rank] in the activation type")
-    _need(a2_bias is None or (a2_bias.dtype == torch.float32 and a2_bias.numel() == heads * dim), "the decay bias must be float32 [heads * dim]")
-    _need(norm_weight is None or (norm_weight.dtype == torch.float32 and norm_weight.numel() == vdim), "the norm weight must be float32 [vdim]")
-    _need(state.dtype == torch.float32 and tuple(state.shape[1:]) == (heads, dim, vdim), "the state must be float32 [slots, heads, dim, vdim]")
+    _gpu(proj, a2, a2_bias, norm_weight, state, state_slots, cu_q, seg_items, req_first, bonus, decay_input)
+    T, width, offs, tail = _recurrence_operands(proj, q_off, k_off, v_off, g_off, u_off, a2, a2_bias, norm_weight, state, heads,
+                                                dim, vdim, decay, bonus, decay_input)
     _i32(state_slots, n_requests, "state_slots")
     _i32(cu_q, n_requests + 1, "cu_q")
     _i32(seg_items, 4 * n_segments, "seg_items")
@@ -1494,11 +1535,64 @@ def linear_recurrence_segments(proj, q_off: int, k_off: int, v_off: int, g_off: 
     workspace = torch.empty(max(int(need), 1), dtype=torch.float32, device=proj.device)
     out = torch.empty((T, heads * vdim), dtype=proj.dtype, device=proj.device)
     _check(lib.cw_linear_recurrence_segments(
-        dtype_code(proj.dtype), _ptr(proj), width, q_off, k_off, v_off, g_off, u_off, _ptr(a2), _ptr(a2_bias),
+        dtype_code(proj.dtype), _ptr(proj), width, *offs, _ptr(a2), _ptr(a2_bias),
         _ptr(norm_weight), _ptr(state), state.shape[0], _ptr(state_slots), _ptr(cu_q), _ptr(seg_items), n_segments,
         int(seg_tokens), _ptr(req_first), _ptr(workspace), _ptr(out), n_requests, T, heads, dim, vdim, a2.shape[1], float(q_scale),
-        1.0 / float(tau), float(eps), _stream()), "linear_recurrence_segments")
+        1.0 / float(tau), float(eps), *tail, _stream()), "linear_recurrence_segments")
     return out
+
+
+SHIFT_MIX_TOKENS = 16   # tokens of one request that a work item of ``shift_mix`` holds
+
+
+def shift_mix(x: torch.Tensor, mu: torch.Tensor, state: torch.Tensor, prev_off: int, state_slots, cu_q, items,
+              n_items: int) -> torch.Tensor:
+    """[n, T, W]: out[s, t] = x[t] + (before[t] - x[t]) * mu[s], ``before`` the row of the request's
+    token one position earlier: the row above, or for the first token of a request's portion the
+    W floats that the request's slot of ``state`` (float32 [slots, ...]) holds from ``prev_off``
+    (zeros in a fresh slot). The portion's last row is then left there for the next step. ``mu``
+    [n, W]; ``items`` int32 [n_items, 4]: (request, first token, tokens, 0), a request's first item
+    beginning at its token 0, at most ``SHIFT_MIX_TOKENS`` tokens each."""
+    _gpu(x, mu, state, state_slots, cu_q, items)
+    T, W = x.shape
+    _need(x.is_contiguous() and mu.dim() == 2 and mu.shape[1] == W and mu.is_contiguous(), "mu must be [n, W]")
+    _need(state.dtype == torch.float32 and state.dim() >= 2 and state.is_contiguous() and 0 <= prev_off
+          and prev_off + W <= state[0].numel(), "the state must be float32 [slots, >= prev_off + W]")
+    R = state_slots.numel()
+    _i32(state_slots, R, "state_slots")
+    _i32(cu_q, R + 1, "cu_q")
+    _i32(items, 4 * n_items, "items")
+    out = torch.empty((mu.shape[0], T, W), dtype=x.dtype, device=x.device)
+    _check(_load("rowwise").cw_shift_mix(_ptr(x), dtype_code(x.dtype), _ptr(mu), dtype_code(mu.dtype), mu.shape[0], _ptr(state),
+                                         state[0].numel(), int(prev_off), state.shape[0], _ptr(state_slots), _ptr(cu_q),
+                                         _ptr(items), int(n_items), _ptr(out), T, W, _stream()), "shift_mix")
+    return out
+
+
+def stream_beside_input(resid: torch.Tensor, pending, model_input: torch.Tensor, dtype, extra: int = 0, hot: int = -1) -> torch.Tensor:
+    """Adds what is still ``pending`` (None, a tensor, a :class:`PendingPair` or
+    :class:`PartialSums`) to the float32 stream ``resid`` in place and returns [T, 2 H + extra] in
+    ``dtype``: the stream beside the model's input (float32 [T, H]), then ``extra`` columns of
+    zeros with a one in column ``hot`` (which lets the product that follows add one of ``extra``
+    learned rows exactly, in its own float32 sums)."""
+    a = b = None
+    if isinstance(pending, PendingPair):
+        a, b = pending.first, pending.second
+    elif pending is not None:
+        a = pending
+    a = a.sum(dtype) if isinstance(a, PartialSums) else a
+    b = b.sum(dtype) if isinstance(b, PartialSums) else b
+    _gpu(resid, a, b, model_input)
+    T, H = resid.shape
+    _need(resid.dtype == torch.float32 and model_input.dtype == torch.float32 and tuple(model_input.shape) == (T, H)
+          and resid.is_contiguous() and model_input.is_contiguous(), "stream and input must be float32 [T, H]")
+    for t in (a, b):
+        _need(t is None or (tuple(t.shape) == (T, H) and t.dtype == dtype and t.is_contiguous()), "a pending output must be [T, H] in the activation type")
+    _need(extra >= 0 and -1 <= hot < max(extra, 1), "the one must lie inside the extra columns")
+    image = torch.empty((T, 2 * H + extra), dtype=dtype, device=resid.device)
+    _check(_load("rowwise").cw_stream_beside_input(_ptr(resid), _ptr(a), _ptr(b), _ptr(model_input), _ptr(image), dtype_code(dtype),
+                                                   T, H, int(extra), int(hot), _stream()), "stream_beside_input")
+    return image
 
 
 SINK_DECODE_MAX_RUN = 128
@@ -1637,14 +1731,16 @@ def gelu_erf_(x: torch.Tensor) -> torch.Tensor:
     return x
 
 
-def sigmoid_mul_(a: torch.Tensor, z: torch.Tensor, z_off: int) -> torch.Tensor:
-    """a[t, j] <- a[t, j] * sigmoid(z[t, z_off + j]), in place on ``a`` [T, n]; ``z`` [T, width]."""
+def sigmoid_mul_(a: torch.Tensor, z: torch.Tensor, z_off: int, group: int = 1) -> torch.Tensor:
+    """a[t, j] <- a[t, j] * sigmoid(z[t, z_off + j // group]), in place on ``a`` [T, n]; ``z``
+    [T, width]. ``group`` 1: a gate an element; g: one gate for every run of g elements (a head)."""
     _gpu(a, z)
     T, n = a.shape
-    _need(z.dim() == 2 and z.shape[0] == T and z.dtype == a.dtype and 0 <= z_off and z_off + n <= z.shape[1],
+    _need(group >= 1 and n % group == 0, "the gated runs must tile the row")
+    _need(z.dim() == 2 and z.shape[0] == T and z.dtype == a.dtype and 0 <= z_off and z_off + n // group <= z.shape[1],
           "the gates must be [T, width] columns of the activations' type")
-    _check(_load("rowwise").cw_sigmoid_mul(_ptr(a), _ptr(z), dtype_code(a.dtype), z.shape[1], int(z_off), T, n, _stream()),
-           "sigmoid_mul")
+    _check(_load("rowwise").cw_sigmoid_mul(_ptr(a), _ptr(z), dtype_code(a.dtype), z.shape[1], int(z_off), T, n, int(group),
+                                           _stream()), "sigmoid_mul")
     return a
 
 
@@ -1772,7 +1868,8 @@ def heads_linear(x: torch.Tensor, weight: torch.Tensor, out: torch.Tensor) -> to
 def rows_attention(q, q_strides, out, out_strides, k_plane, v_plane, block_tables, ctx_lens, cu_q, items, n_items: int,
                    heads: int, kv_heads: int, dim: int, vdim: int, block_size: int, scale: float, maps: int = 1,
                    mask: str = "causal", mask_size: int = 0, sink=None, lam=None, head_norm_eps=None,
-                   post_mult: float = 1.0, mfma: bool = False, key_runs: int = 1) -> None:
+                   post_mult: float = 1.0, mfma: bool = False, key_runs: int = 1, keep_first: int = 0,
+                   softcap: float = 0.0) -> None:
     """Softmax attention of the step's queries over paged rows. Query (t, head, map, d) lies at
     ``q.flatten()[t * q_strides[0] + head * q_strides[1] + map * dim + d]``, output (t, head, c) at
     ``out.flatten()[t * out_strides[0] + head * out_strides[1] + c]`` (token-major or head-major
@@ -1781,6 +1878,8 @@ def rows_attention(q, q_strides, out, out_strides, k_plane, v_plane, block_table
     the values are the first ``vdim`` elements of the key row (``maps`` 1).
     ``mask``: "causal", "window" (the ``mask_size`` latest positions) or "segments" (the earlier
     tokens of the token's segment of ``mask_size`` positions, segments counted from position 0).
+    ``keep_first`` n (with a window): the request's first n positions stay visible to every later
+    token. ``softcap`` c > 0: scores are squashed, c * tanh(scale * q . k / c), before the softmax.
     ``sink`` float32 [heads]: exp(sink) joins the denominator. ``maps`` 2: the head's output is
     map 0 minus ``lam`` (one float32 element) times map 1. ``head_norm_eps`` not None: the head's
     output is divided by its root mean square and multiplied by ``post_mult``. ``items`` int32
@@ -1818,7 +1917,10 @@ def rows_attention(q, q_strides, out, out_strides, k_plane, v_plane, block_table
     _need((maps == 1 and lam is None) or (maps == 2 and lam is not None and lam.dtype == torch.float32 and lam.numel() == 1),
           "two maps take one float32 lambda, one map none")
     _need(mask in MASK_KINDS and (mask == "causal" or mask_size >= 1), f"mask {mask!r} of size {mask_size}")
+    _need(keep_first >= 0 and (keep_first == 0 or mask == "window"), "first positions are kept visible behind a window only")
+    _need(softcap >= 0.0, "a score cap is positive (0: none)")
     if mfma:
+        _need(keep_first == 0 and softcap == 0.0, "the matrix-core kernel has no kept first positions and no score cap")
         lib = _load("rows_attention")
         _need(rows_mfma_supported(dim, vdim, maps, q.dtype, alias), "the matrix-core kernel does not take this geometry")
         need = int(lib.cw_rows_mfma_workspace_floats(n_items, heads, kv_heads, maps, dim, vdim, int(alias), key_runs))
@@ -1834,7 +1936,8 @@ def rows_attention(q, q_strides, out, out_strides, k_plane, v_plane, block_table
         dtype_code(q.dtype), _ptr(q), qs, qh, _ptr(out), os_, oh, _ptr(k_plane), _ptr(k_plane if alias else v_plane), k2.shape[1],
         v_row, rows, _ptr(block_tables), block_tables.shape[1], _ptr(ctx_lens), _ptr(cu_q), _ptr(items), n_items, _ptr(sink),
         _ptr(lam), heads, kv_heads, dim, vdim, maps, block_size, MASK_KINDS[mask], int(mask_size), float(scale),
-        0 if head_norm_eps is None else 1, float(head_norm_eps or 0.0), float(post_mult), _stream()), "rows_attention")
+        0 if head_norm_eps is None else 1, float(head_norm_eps or 0.0), float(post_mult), int(keep_first), float(softcap),
+        _stream()), "rows_attention")
 
 
 # ---------------------------------------------------------------------------------------------
@@ -1884,9 +1987,14 @@ def stream_norm(resid, weight, weight_offset: float, eps: float, out, rows=None)
     return out
 
 
+HEAD_PAIRINGS = {"halves": 0, "neighbours": 1}
+HEAD_NORMS = {"none": 0, "before": 1, "after": 2}
+
+
 def headnorm_rope_store(proj: torch.Tensor, q_off: int, k_off: int, v_off: int, n_q_vectors: int, n_k_vectors: int, dim: int,
                         nv: int, bias, q_weight, k_weight, eps: float, positions, freq, rot_dims: int, slots, k_plane,
-                        v_plane, values_from_keys: bool = False) -> None:
+                        v_plane, values_from_keys: bool = False, pairing: str = "halves", norm=None,
+                        query_temperature=None) -> None:
     """Rows of ``proj`` [T, width] hold a token's query vectors (``n_q_vectors`` of ``dim`` elements
     from column q_off), key vectors (``n_k_vectors`` from k_off) and value projection (``nv``
     elements from v_off). ``bias`` ([width] or None) is added; every query and key vector by itself
@@ -1895,7 +2003,13 @@ def headnorm_rope_store(proj: torch.Tensor, q_off: int, k_off: int, v_off: int, 
     angle = position * freq[i], ``freq`` float32 [rot_dims / 2]). Queries are rewritten in place,
     keys go to ``k_plane[slots[t]]``, values to ``v_plane[slots[t]]``: the biased value projection,
     or with ``values_from_keys`` the biased key projection before norm and rotation. ``slots``
-    None or a negative slot: no cache row is written."""
+    None or a negative slot: no cache row is written.
+
+    ``pairing`` "neighbours": elements 2i and 2i + 1 turn together by freq[i] (instead of i and
+    i + rot_dims / 2). ``norm``: "before" (the norm, then the rotation), "after" (the rotated vector is
+    divided by its own root mean square), "none"; None: "before" if weights are given, else
+    "none". The weights may be absent with either norm. ``query_temperature`` (coef, every): every
+    query is multiplied, last, by 1 + coef * ln(floor((position + 1) / every) + 1)."""
     _gpu(proj, bias, q_weight, k_weight, positions, freq, slots, k_plane, v_plane)
     T, width = proj.shape
     if positions is not None:
@@ -1908,6 +2022,12 @@ def headnorm_rope_store(proj: torch.Tensor, q_off: int, k_off: int, v_off: int, 
         _need(q_weight.numel() == dim and k_weight.numel() == dim and q_weight.dtype == k_weight.dtype, "norm weights must be [dim]")
     _need(rot_dims == 0 or (freq is not None and positions is not None and freq.dtype == torch.float32
                             and freq.numel() >= rot_dims // 2), "freq must be float32 with rot_dims / 2 elements")
+    _need(pairing in HEAD_PAIRINGS, f"pairing {pairing!r}: expected one of {sorted(HEAD_PAIRINGS)}")
+    if norm is None:
+        norm = "before" if q_weight is not None else "none"
+    _need(norm in HEAD_NORMS and (norm != "none" or q_weight is None), f"norm {norm!r}: 'before', 'after' or 'none' (which takes no weights)")
+    coef, every = query_temperature if query_temperature is not None else (0.0, 0)
+    _need(int(every) >= 0 and (int(every) == 0 or positions is not None), "a query temperature needs positions and a positive period")
     rows = 0
     if slots is not None:
         nk = n_k_vectors * dim
@@ -1919,7 +2039,8 @@ def headnorm_rope_store(proj: torch.Tensor, q_off: int, k_off: int, v_off: int, 
         _ptr(proj), dtype_code(proj.dtype), width, int(q_off), int(k_off), int(v_off), int(n_q_vectors), int(n_k_vectors), int(dim),
         int(nv), _ptr(bias), dtype_code(bias.dtype) if bias is not None else 0, _ptr(q_weight), _ptr(k_weight),
         dtype_code(q_weight.dtype) if q_weight is not None else 0, float(eps), _ptr(positions), _ptr(freq), int(rot_dims),
-        _ptr(slots), _ptr(k_plane), _ptr(v_plane), int(bool(values_from_keys)), rows, T, _stream()), "headnorm_rope_store")
+        _ptr(slots), _ptr(k_plane), _ptr(v_plane), int(bool(values_from_keys)), rows, T, HEAD_PAIRINGS[pairing], HEAD_NORMS[norm],
+        float(coef), int(every), _stream()), "headnorm_rope_store")
 
 
 def relu_squared_(x: torch.Tensor) -> torch.Tensor:
@@ -1968,20 +2089,34 @@ def scale_(x: torch.Tensor, s: float) -> torch.Tensor:
 ROUTER_KINDS = {"sigmoid": 0, "softmax": 1}
 
 
-def moe_route(x: torch.Tensor, router: torch.Tensor, top: int, kind: str = "sigmoid", renormalize: bool = False):
+def moe_route(x: torch.Tensor, router: torch.Tensor, top: int, kind: str = "sigmoid", renormalize: bool = False,
+              correction=None, groups=None, extra: int = 0, renorm_eps: float = 0.0):
     """(choice int32 [T, top], score float32 [T, top]): the ``top`` experts with the largest
     logistic (or softmax) of router x, the lower index first among equals, in falling order;
-    ``renormalize``: the chosen scores are divided by their sum. float32 sums."""
-    _gpu(x, router)
+    ``renormalize``: the chosen scores are divided by their sum (plus ``renorm_eps``). float32 sums.
+
+    ``correction`` float32 [experts]: added to the scores for the choice only. ``groups``
+    (count, kept, top): the experts lie in ``count`` equal runs of neighbours, a run's score is the
+    sum of its ``top`` largest choice scores, and only experts of the ``kept`` best runs can be
+    chosen. ``extra`` n: the router's matrix has n more rows behind the experts' (gates that
+    read the same input); their logistic values come back as a third result, float32 [T, n]."""
+    _gpu(x, router, correction)
     T, H = x.shape
-    E = router.shape[0]
-    _need(router.dim() == 2 and router.shape[1] == H and router.dtype == x.dtype, "the router must be [experts, H] in x's type")
+    E = router.shape[0] - int(extra)
+    _need(router.dim() == 2 and router.shape[1] == H and router.dtype == x.dtype and extra >= 0 and E >= 1,
+          "the router must be [experts (+ extra), H] in x's type")
     _need(1 <= top <= E and kind in ROUTER_KINDS, f"top {top} of {E} experts, router kind {kind!r}")
+    _need(correction is None or (correction.dtype == torch.float32 and correction.numel() == E), "the correction must be float32 [experts]")
+    count, kept, run_top = groups if groups is not None else (1, 1, 1)
+    _need(count >= 1 and E % count == 0 and 1 <= kept <= count and run_top >= 1 and (E // count) * kept >= top,
+          f"{E} experts in {count} runs of which {kept} are kept cannot give {top} experts")
     choice = torch.empty((T, top), dtype=torch.int32, device=x.device)
     score = torch.empty((T, top), dtype=torch.float32, device=x.device)
+    gates = torch.empty((T, extra), dtype=torch.float32, device=x.device) if extra else None
     _check(_load("moe").cw_moe_route(_ptr(x), _ptr(router), dtype_code(x.dtype), T, H, E, top, ROUTER_KINDS[kind],
-                                     int(bool(renormalize)), _ptr(choice), _ptr(score), _stream()), "moe_route")
-    return choice, score
+                                     int(bool(renormalize)), _ptr(choice), _ptr(score), _ptr(correction), int(count), int(kept),
+                                     int(run_top), int(extra), _ptr(gates), float(renorm_eps), _stream()), "moe_route")
+    return (choice, score, gates) if extra else (choice, score)
 
 
 MOE_KERNELS = {"plain": 0, "stream": 1, "wide": 2, "grouped": 3}
@@ -2091,10 +2226,20 @@ def moe_down(inner: torch.Tensor, down: torch.Tensor, plan: ExpertRows, score: t
     return out
 
 
-def moe_combine(y: torch.Tensor, top: int, out: torch.Tensor) -> torch.Tensor:
-    """out[t] = y[t * top] + ... + y[t * top + top - 1], added in that order in float32."""
-    _gpu(y, out)
+def moe_combine(y: torch.Tensor, top: int, out: torch.Tensor, always=None, always_gate=None) -> torch.Tensor:
+    """out[t] = y[t * top] + ... + y[t * top + top - 1], added in that order in float32; then
+    ``always`` [T, H] (the output of an expert that every token uses) joins, times
+    ``always_gate[t, 0]`` (float32 [T, n]) if given."""
+    _gpu(y, out, always, always_gate)
     T, H = out.shape
     _need(tuple(y.shape) == (T * top, H) and y.dtype == out.dtype, "y must be [T * top, H]")
-    _check(_load("moe").cw_moe_combine(_ptr(y), _ptr(out), dtype_code(out.dtype), T, top, H, _stream()), "moe_combine")
+    _need(always is None or (tuple(always.shape) == (T, H) and always.dtype == out.dtype and always.is_contiguous()),
+          "the expert of every token must be [T, H] in the output's type")
+    stride = 0
+    if always_gate is not None:
+        _need(always is not None and always_gate.dtype == torch.float32 and always_gate.dim() == 2 and always_gate.shape[0] == T
+              and always_gate.is_contiguous(), "the gate must be float32 [T, n]")
+        stride = always_gate.shape[1]
+    _check(_load("moe").cw_moe_combine(_ptr(y), _ptr(out), dtype_code(out.dtype), T, top, H, _ptr(always), _ptr(always_gate),
+                                       int(stride), _stream()), "moe_combine")
     return out

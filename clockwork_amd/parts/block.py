@@ -120,6 +120,51 @@ class ParallelBlock:
         return None
 
 
+class TwoNormParallelBlock:
+    """x = x + mixer(norm1(x)) + ffn(norm2(x)): mixer and feed-forward side by side, each behind a
+    norm of its own of the same x; the feed-forward and its norm may be absent.
+
+    The residual stream is float32. Both outputs are handed on unadded (``ops.PendingPair``) when
+    the norm that comes next adds them inside its kernel; else the block adds them itself. The
+    first norm takes what the block before left pending; the second then norms the same, updated
+    stream."""
+
+    def __init__(self, mixer, mixer_norm, feed_forward=None, ffn_norm=None) -> None:
+        if (feed_forward is None) != (ffn_norm is None):
+            raise ValueError("a block has a feed-forward and its norm, or neither")
+        self.mixer, self.mixer_norm, self.feed_forward, self.ffn_norm = mixer, mixer_norm, feed_forward, ffn_norm
+
+    def parts(self) -> dict:
+        parts = {"mixer": self.mixer}
+        if self.feed_forward is not None:
+            parts["feed_forward"] = self.feed_forward
+        parts["mixer_norm"] = self.mixer_norm
+        if self.ffn_norm is not None:
+            parts["ffn_norm"] = self.ffn_norm
+        return parts
+
+    def first_norm(self):
+        return self.mixer_norm
+
+    def forward(self, resid, delta, ctx, cache):
+        both = getattr(self.mixer_norm, "forward_pair", None)
+        if self.feed_forward is not None and both is not None:
+            x, y = both(resid, delta, self.ffn_norm)   # one kernel: the two norms share the row's statistics
+        else:
+            x = self.mixer_norm.forward(resid, delta)
+            y = self.ffn_norm.forward(resid, None) if self.feed_forward is not None else None
+        a = self.mixer.forward(x, ctx, cache)
+        if self.feed_forward is None:
+            return a
+        b = self.feed_forward.forward(y, ctx)
+        if isinstance(a, ops.PartialSums):
+            a = a.sum(x.dtype)
+        if getattr(ctx, "next_norm_accepts_pending", False):
+            return ops.PendingPair(a, b)
+        ops.gated_residual_add(resid, ops.GatedBranches(None, None, a, b))
+        return None
+
+
 class BranchNormBlock:
     """x = x + c * N1(mixer(x)); x = x + c * N2(ffn(x)): mixer and feed-forward read the stream
     itself, and what is normed is their output (``BranchRMSNorm``, whose spec holds c). The

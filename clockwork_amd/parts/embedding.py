@@ -122,3 +122,42 @@ class LinearHead(Part):
 
     def kernel_libraries(self) -> list:
         return [("rowwise", None)] if self.spec.softcap is not None or self.spec.scale is not None else []
+
+
+class StreamReentry(Part):
+    """The stream made anew from itself and the model's input before a pass of a repeated run of
+    layers (``StreamReentrySpec``): x <- R [x; x0] + s_n.
+
+    One kernel adds what the block before left pending to the float32 stream and writes
+    [x, x0, e_n] in the activation type, e_n a one in column n of a few extra columns; one product
+    with [R | s^T] then yields R [x; x0] + s_n with the learned row inside the product's float32
+    sums. The result is the new float32 stream."""
+
+    graph_safe = True
+
+    def __init__(self, spec) -> None:
+        self.spec = spec
+        self.extra = -(-spec.passes // 8) * 8   # the operand's rows stay a multiple of 16 bytes
+
+    def param_specs(self):
+        H = self.spec.hidden_size
+        return {"in_weight": ParamSpec((H, 2 * H), init=("normal", 0.7 / (2 * H) ** 0.5 * 2 ** 0.5)),
+                "step": ParamSpec((self.spec.passes, H), init=("normal", 0.1))}
+
+    def kernel_libraries(self) -> list:
+        return [("rowwise", None)]
+
+    def bind(self, params, device, dtype) -> None:
+        H, P = self.spec.hidden_size, self.spec.passes
+        weight = torch.zeros((H, 2 * H + self.extra), dtype=dtype, device=device)
+        weight[:, : 2 * H] = params["in_weight"]
+        weight[:, 2 * H : 2 * H + P] = params["step"].to(dtype).t()
+        self.weight = weight
+        self.dtype = dtype
+
+    def forward(self, resid: torch.Tensor, pending, model_input: torch.Tensor, pass_no: int, ctx) -> torch.Tensor:
+        """The new float32 stream [T, hidden]; ``pending`` has joined the old one on the way."""
+        if not 0 <= pass_no < self.spec.passes:
+            raise ValueError(f"pass {pass_no} of {self.spec.passes}")
+        image = ops.stream_beside_input(resid, pending, model_input, self.dtype, self.extra, pass_no)
+        return ops.linear(image, self.weight, out_dtype=torch.float32, policy=getattr(ctx, "products", None))

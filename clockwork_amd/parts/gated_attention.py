@@ -12,7 +12,10 @@ given back while the request runs.
 
 bfloat16 steps whose head size the kernels for plain grouped attention are built for run on
 those (the two planes have the layout of a key/value cache); everything else, float32 included,
-on the kernel for paged rows.
+on the kernel for paged rows, which is also the one that knows kept first positions behind a
+window and a cap on the scores. The norm may come before or after the rotation and may lack
+weights, the rotation may pair halves or neighbours, queries may carry a factor that grows with
+the logarithm of their position, and the gate may be one number a head: all in the same kernels.
 """
 
 from __future__ import annotations
@@ -24,7 +27,7 @@ from clockwork_amd.config.spec import PagedRowsSpec, ParamSpec
 from clockwork_amd.parts.attention import attention_plan
 from clockwork_amd.parts.base import EntryCache, Part
 from clockwork_amd.parts.sink_attention import query_runs
-from clockwork_amd.parts.specs import GatedAttentionSpec
+from clockwork_amd.parts.specs import GatedAttentionSpec, RopePairsSpec
 
 
 class GatedAttention(Part):
@@ -40,7 +43,8 @@ class GatedAttention(Part):
         # columns of the fused product: queries, keys, values (if projected), gate (if any)
         self.v_off = self.q_width + self.k_width
         self.g_off = self.v_off + (self.v_width if self.own_values else 0)
-        self.in_width = self.g_off + (self.out_width if spec.output_gate else 0)
+        self.gate_width = 0 if not spec.output_gate else (spec.num_heads if spec.gate_per_head else self.out_width)
+        self.in_width = self.g_off + self.gate_width
 
     def param_specs(self):
         s = self.spec
@@ -52,21 +56,22 @@ class GatedAttention(Part):
             specs["in_bias"] = ParamSpec((self.in_width,), precision="stored", init=("normal", 0.02))
         if s.out_bias:
             specs["out_bias"] = ParamSpec((s.hidden_size,), precision="compute", init=("normal", 0.02))
-        if s.qk_norm:
+        if s.qk_norm and s.qk_norm_weight:
             specs["q_norm"] = ParamSpec((s.key_dim,), precision="stored", init=("one_plus_uniform", 0.3))
             specs["k_norm"] = ParamSpec((s.key_dim,), precision="stored", init=("one_plus_uniform", 0.3))
         return specs
 
     def cache_need(self):
         s = self.spec
-        return PagedRowsSpec((("k", (s.num_kv_heads, s.key_dim)), ("v", (s.num_kv_heads, s.value_dim))), window=s.window)
+        return PagedRowsSpec((("k", (s.num_kv_heads, s.key_dim)), ("v", (s.num_kv_heads, s.value_dim))), window=s.window,
+                             keep_first=s.keep_first)
 
     def _plain_kernels(self, dtype) -> bool:
         """Do the kernels for plain grouped attention take these heads? bfloat16, keys and values
         of one size that they are built for."""
         s = self.spec
         return (dtype == torch.bfloat16 and s.key_dim == s.value_dim and s.key_dim % 32 == 0 and 32 <= s.key_dim <= 256
-                and self.in_width % 8 == 0)
+                and self.in_width % 8 == 0 and not s.keep_first and s.softcap is None)
 
     def kernel_libraries(self) -> list:
         # the library of plain grouped attention is loaded (and, if missing, built) when the part is
@@ -79,6 +84,8 @@ class GatedAttention(Part):
         self.out_weight, self.out_bias = params["out_weight"], params.get("out_bias")
         self.q_norm, self.k_norm = params.get("q_norm"), params.get("k_norm")
         self.rot_dims = s.position.rotary_dim if s.position is not None else 0
+        self.pairing = "neighbours" if isinstance(s.position, RopePairsSpec) else "halves"
+        self.norm_order = "none" if not s.qk_norm else ("after" if s.qk_norm_after_rotation else "before")
         self.freq = None
         if self.rot_dims:
             # base^(-2i / n), made on the host in float64 and rounded once
@@ -112,7 +119,8 @@ class GatedAttention(Part):
         proj = ops.linear(x, self.in_weight, policy=policy)
         ops.headnorm_rope_store(proj, 0, self.q_width, self.v_off, s.num_heads, s.num_kv_heads, s.key_dim, self.v_width,
                                 self.in_bias, self.q_norm, self.k_norm, s.norm_eps, ctx.positions, self.freq, self.rot_dims,
-                                ctx.slots[cache.group], k_plane, v_plane, values_from_keys=not self.own_values)
+                                ctx.slots[cache.group], k_plane, v_plane, values_from_keys=not self.own_values,
+                                pairing=self.pairing, norm=self.norm_order, query_temperature=s.query_temperature)
         out = torch.empty((x.shape[0], self.out_width), dtype=x.dtype, device=x.device)
         if self.plain:
             self._attend_plain(proj, out, ctx, cache, k_plane, v_plane)
@@ -121,12 +129,13 @@ class GatedAttention(Part):
             ops.rows_attention(proj, (proj.shape[1], s.key_dim), out, (out.shape[1], s.value_dim), k_plane, v_plane,
                                ctx.block_tables[cache.group], ctx.ctx_lens, ctx.cu_q, items, n_items, s.num_heads, s.num_kv_heads,
                                s.key_dim, s.value_dim, cache.block_size, s.scale, maps=1,
-                               mask="window" if s.window is not None else "causal", mask_size=s.window or 0)
+                               mask="window" if s.window is not None else "causal", mask_size=s.window or 0,
+                               keep_first=s.keep_first, softcap=s.softcap or 0.0)
         if s.output_gate:
             bias_free = self.in_bias is None
             if not bias_free:
                 raise NotImplementedError("an output gate with a bias")
-            ops.sigmoid_mul_(out, proj, self.g_off)
+            ops.sigmoid_mul_(out, proj, self.g_off, group=s.value_dim if s.gate_per_head else 1)
         return ops.linear(out, self.out_weight, self.out_bias, policy=policy)
 
     def _attend_plain(self, q, out, ctx, cache, k_plane, v_plane) -> None:

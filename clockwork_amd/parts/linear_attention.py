@@ -109,3 +109,94 @@ class DecayedLinearAttention(Part):
         else:
             out = ops.linear_recurrence(*common, *sizes)
         return ops.linear(out, self.out_weight, policy=policy)
+
+
+class ShiftedRecurrence(Part):
+    """A matrix recurrence a head whose inputs are mixes of a token with the one before it
+    (``ShiftedRecurrenceSpec``).
+
+    One kernel makes the five mixes of the step's tokens (the row before a portion's first token
+    waits in the request's state slot, and the portion's last row is left there); the products
+    for r, k, v and the gate are one batched product over four planes, the decay's low-rank input
+    a product of its own; the recurrence kernels of :class:`DecayedLinearAttention` walk the tokens
+    in their other form (the decay exp(-exp(.)) with tanh on its input, the output read from the
+    state before the token joins it, the token itself through the bonus), norm every head's output
+    with the head's own weights and gate it; output product. Long portions are cut into segments
+    that are walked side by side, as there. A request's slot is float32
+    [heads * dim * dim + hidden]: the matrices, then the last input row."""
+
+    graph_safe = True
+    MIXES = ("r", "k", "v", "g", "w")
+
+    def __init__(self, spec) -> None:
+        self.spec = spec
+        self.inner = spec.num_heads * spec.head_dim
+
+    def param_specs(self):
+        s = self.spec
+        return {
+            # the mixing vectors of r, k, v, g, w one behind the other
+            "mix": ParamSpec((len(self.MIXES) * s.hidden_size,), precision="float32", init=("uniform", 0.0, 1.0)),
+            "rkvg_weight": ParamSpec((4 * self.inner, s.hidden_size)),
+            "decay_in_weight": ParamSpec((s.decay_rank, s.hidden_size), init=("normal", 0.1)),
+            "decay_weight": ParamSpec((self.inner, s.decay_rank), init=("normal", 0.5)),
+            "decay_bias": ParamSpec((self.inner,), precision="float32", init=("uniform", -3.0, 0.5)),
+            "bonus": ParamSpec((s.num_heads, s.head_dim), precision="float32", init=("normal", 0.5)),
+            "norm_weight": ParamSpec((self.inner,), precision="float32", init=("one_plus_uniform", 0.1)),
+            "out_weight": ParamSpec((s.hidden_size, self.inner)),
+        }
+
+    def cache_need(self):
+        s = self.spec
+        return StateSpec((s.num_heads * s.head_dim * s.head_dim + s.hidden_size,), "float32")
+
+    def kernel_libraries(self) -> list:
+        return [("linear_recurrence", None), ("rowwise", None)]
+
+    def bind(self, params, device, dtype) -> None:
+        s = self.spec
+        if not ops.linear_recurrence_supported(s.head_dim, s.head_dim):
+            raise ValueError(f"a state of {s.head_dim} x {s.head_dim} a head is beyond the recurrence kernel "
+                             "(head_dim up to 256)")
+        self.segments_ok = ops.linear_recurrence_segments_supported(s.head_dim, s.head_dim)
+        self.mix = params["mix"].view(len(self.MIXES), s.hidden_size)
+        self.rkvg = params["rkvg_weight"].view(4, self.inner, s.hidden_size)
+        self.decay_in = params["decay_in_weight"]
+        self.decay_weight, self.decay_bias = params["decay_weight"], params["decay_bias"]
+        self.bonus, self.norm_weight = params["bonus"], params["norm_weight"]
+        self.out_weight = params["out_weight"]
+
+    def _items(self, ctx):
+        from clockwork_amd.parts.sink_attention import query_runs
+
+        return query_runs(ctx, ops.SHIFT_MIX_TOKENS)
+
+    _segments = DecayedLinearAttention._segments
+
+    def prepare(self, ctx) -> None:
+        self._items(ctx)
+        self._segments(ctx)
+
+    def shape_class(self, q_lens, ctx_lens):
+        return "segments" if max(q_lens, default=0) > SEGMENT_MIN_TOKENS and self.segments_ok else "token by token"
+
+    def forward(self, x: torch.Tensor, ctx, cache: EntryCache) -> torch.Tensor:
+        s = self.spec
+        policy = getattr(ctx, "products", None)
+        T = x.shape[0]
+        state = cache.state
+        items, n_items = self._items(ctx)
+        mixes = ops.shift_mix(x, self.mix, state, s.num_heads * s.head_dim * s.head_dim, ctx.state_slots, ctx.cu_q, items, n_items)
+        planes = torch.empty((4, T, self.inner), dtype=x.dtype, device=x.device)
+        ops.heads_linear(mixes[:4], self.rkvg, planes)
+        decay_input = ops.linear(mixes[4], self.decay_in, policy=policy)
+        common = (planes, 0, 1, 2, 3, 0, self.decay_weight, self.decay_bias, self.norm_weight, state, ctx.state_slots, ctx.cu_q)
+        sizes = (ctx.num_requests, s.num_heads, s.head_dim, s.head_dim, 1.0, 1.0, s.norm_eps)
+        form = dict(decay="double_exp", bonus=self.bonus, decay_input=decay_input)
+        plan = self._segments(ctx)
+        if plan is not None:
+            seg_items, n_segments, first = plan
+            out = ops.linear_recurrence_segments(*common, seg_items, n_segments, SEGMENT_TOKENS, first, *sizes, **form)
+        else:
+            out = ops.linear_recurrence(*common, *sizes, **form)
+        return ops.linear(out, self.out_weight, policy=policy)

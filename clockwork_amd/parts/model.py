@@ -34,9 +34,11 @@ def _build_layers(spec: ModelSpec) -> list:
     ]
 
 
-def _named_parts(embedding, layers, final_norm, head) -> list:
+def _named_parts(embedding, layers, final_norm, head, reentry=None) -> list:
     """(prefix of its parameters' names, part) for every part of the model."""
     named = [("embed.", embedding)]
+    if reentry is not None:
+        named.append(("reentry.", reentry))
     for i, layer in enumerate(layers):
         named += [(f"layers.{i}.{role}.", part) for role, part in layer.parts().items()]
     named += [("final_norm.", final_norm), ("lm_head.", head)]
@@ -46,7 +48,7 @@ def _named_parts(embedding, layers, final_norm, head) -> list:
 def model_param_specs(spec: ModelSpec) -> dict[str, ParamSpec]:
     """Every tensor the model owns, by its internal name. Needs no GPU."""
     named = _named_parts(build_part(_embedding_spec(spec)), _build_layers(spec), build_part(spec.final_norm),
-                         build_part(_head_spec(spec)))
+                         build_part(_head_spec(spec)), build_part(spec.reentry) if spec.reentry is not None else None)
     return {prefix + name: p for prefix, part in named for name, p in part.param_specs().items()}
 
 
@@ -58,6 +60,7 @@ class DecoderModel:
         self.layers = _build_layers(spec)
         self.final_norm = build_part(spec.final_norm)
         self.head = build_part(_head_spec(spec))
+        self.reentry = build_part(spec.reentry) if spec.reentry is not None else None
         for i, entry in enumerate(spec.run):
             if entry.add_input:
                 first_norm = getattr(self.layers[entry.layer], "first_norm", None)
@@ -66,7 +69,7 @@ class DecoderModel:
                                      f"layer {entry.layer} cannot take (no accepts_stream_input)")
 
     def named_parts(self) -> list:
-        return _named_parts(self.embedding, self.layers, self.final_norm, self.head)
+        return _named_parts(self.embedding, self.layers, self.final_norm, self.head, self.reentry)
 
     def param_specs(self) -> dict[str, ParamSpec]:
         return {prefix + name: p for prefix, part in self.named_parts() for name, p in part.param_specs().items()}
@@ -155,10 +158,16 @@ class DecoderModel:
         # a run entry that is fed the model's input again needs it as it was: the stream is updated
         # in place, so the embedding part makes it a second time (a gather, and a kernel launch
         # like any other for a step that is captured as a graph)
-        again = self.embedding.forward(ctx) if any(e.add_input for e in self.spec.run) else None
+        again = self.embedding.forward(ctx) if any(e.add_input or e.reenter is not None for e in self.spec.run) else None
         delta = None
         run = self.spec.run
         for i, entry in enumerate(run):
+            if entry.reenter is not None:
+                # the stream is made anew from itself (with what is pending) and the model's input
+                if isinstance(delta, (ops.GatedBranches, ops.StreamImage, ops.WithStreamInput)):
+                    raise TypeError("the stream is re-entered with plain pending outputs only")
+                resid = self.reentry.forward(resid, delta, again, entry.reenter, ctx)
+                delta = None
             if entry.add_input:
                 delta = ops.WithStreamInput(delta, again)
             # may this block hand on two pending outputs? Only if the norm that takes them next (the

@@ -31,6 +31,16 @@ class RopeNeoxSpec:
 
 
 @dataclass(frozen=True)
+class RopePairsSpec:
+    """Rotary position encoding over neighbouring elements: (2i, 2i + 1) turn together by the angle
+    position / theta^(2i / rotary_dim); the first ``rotary_dim`` elements of each head are rotated,
+    the rest pass through."""
+
+    rotary_dim: int
+    theta: float
+
+
+@dataclass(frozen=True)
 class AttentionSpec:
     """Softmax attention with grouped query heads over a paged key/value cache."""
 
@@ -344,7 +354,16 @@ class GatedAttentionSpec:
     * ``output_gate``: the concatenated heads are multiplied by the logistic function of one more
       projection of the mixer's input before the output projection.
     * ``window`` W: a token sees itself and the W - 1 tokens before it; None: all of them.
-    * ``qkv_bias`` / ``out_bias``."""
+    * ``qkv_bias`` / ``out_bias``.
+    * ``qk_norm_weight`` False: the query/key norm has no weights. ``qk_norm_after_rotation``: the
+      vectors are rotated first and the rotated vector is normed.
+    * ``position`` may also be a ``RopePairsSpec`` (neighbouring elements turn together).
+    * ``keep_first`` n (with a window): the first n positions of a request stay visible to every
+      later token, at their true positions.
+    * ``softcap`` c: scores are squashed before the softmax, c * tanh(scale * q . k / c).
+    * ``query_temperature`` (coef, every): the query at position p is multiplied by
+      1 + coef * ln(floor((p + 1) / every) + 1), after its norm.
+    * ``gate_per_head`` (with ``output_gate``): the gate is one number a head, not one an element."""
 
     hidden_size: int
     num_heads: int
@@ -360,6 +379,12 @@ class GatedAttentionSpec:
     output_gate: bool = False
     qkv_bias: bool = False
     out_bias: bool = False
+    qk_norm_weight: bool = True
+    qk_norm_after_rotation: bool = False
+    keep_first: int = 0
+    softcap: Optional[float] = None
+    query_temperature: Optional[tuple] = None
+    gate_per_head: bool = False
 
     def __post_init__(self):
         if self.num_heads < 1 or self.num_kv_heads < 1 or self.num_heads % self.num_kv_heads:
@@ -374,6 +399,51 @@ class GatedAttentionSpec:
             raise ValueError(f"rotary_dim {self.position.rotary_dim} exceeds key_dim {self.key_dim}")
         if self.window is not None and self.window < 1:
             raise ValueError(f"window must be positive, got {self.window}")
+        if self.keep_first < 0 or (self.keep_first and self.window is None):
+            raise ValueError("first positions are kept visible behind a window only, and their number is not negative")
+        if self.softcap is not None and not self.softcap > 0:
+            raise ValueError(f"softcap must be positive, got {self.softcap}")
+        if self.query_temperature is not None and (len(self.query_temperature) != 2 or int(self.query_temperature[1]) < 1):
+            raise ValueError(f"query_temperature is (coef, every) with every >= 1, got {self.query_temperature!r}")
+        if self.gate_per_head and not self.output_gate:
+            raise ValueError("a gate a head is an output gate")
+
+
+@dataclass(frozen=True)
+class ShiftedRecurrenceSpec:
+    """A recurrence over a matrix state a head whose inputs are mixes of a token with the one
+    before it. With h' the mixer's input one position earlier (zeros before a request's first
+    token) each of r, k, v, g, w reads m_s = h + (h' - h) * mu_s. r, k, v = W_s m_s, cut into
+    ``num_heads`` heads of ``head_dim``; gate = silu(W_g m_g); decay d = exp(-exp(w2 tanh(w1 m_w) +
+    w0)), one number a head and key channel, w1 of ``decay_rank`` rows. A head with state S
+    [head_dim, head_dim], zero at a request's start, float32: o = (S + diag(bonus) k v^T)^T r, then
+    S <- diag(d) S + k v^T. Every head's o is divided by its root mean square (``norm_eps``); the
+    concatenated heads are multiplied by a weight and by the gate, and projected back. The state a
+    request keeps is the matrices and the last input row."""
+
+    hidden_size: int
+    num_heads: int
+    head_dim: int
+    decay_rank: int
+    norm_eps: float
+
+    def __post_init__(self):
+        if min(self.hidden_size, self.num_heads, self.head_dim, self.decay_rank) < 1:
+            raise ValueError("hidden_size, heads, head_dim and decay_rank must be positive")
+
+
+@dataclass(frozen=True)
+class StreamReentrySpec:
+    """The stream made anew from itself and the model's input: x <- R [x; x0] + s_n, with x0 what
+    the embedding part made of the step's tokens, R [hidden, 2 hidden] (x's columns first) and s
+    [passes, hidden], n the number of the pass that begins (``RunEntry.reenter``)."""
+
+    hidden_size: int
+    passes: int
+
+    def __post_init__(self):
+        if self.hidden_size < 1 or self.passes < 1:
+            raise ValueError("hidden_size and passes must be positive")
 
 
 @dataclass(frozen=True)
@@ -384,7 +454,14 @@ class RoutedExpertsSpec:
     largest r chosen (compared through their logits, which still differ where two r round to 1;
     the lower index first among equals), divided by their sum if
     ``renormalize``. ``weight_on`` "input": the result is the sum of E_e(r_e x); "output": the sum
-    of r_e E_e(x)."""
+    of r_e E_e(x).
+
+    ``choice_correction``: a learned float32 number an expert joins r for the choice only; the
+    weights stay r. ``groups`` (count, kept, top): the experts lie in ``count`` equal runs of
+    neighbours; a run's score is the sum of its ``top`` largest choice scores and only experts of
+    the ``kept`` best runs can be chosen. ``renorm_eps`` joins the sum that ``renormalize``
+    divides by. ``shared_intermediate`` n: one more expert of inner width n runs for every token
+    and its output is added, times logistic(w_sg x) (one number a token) if ``shared_gate``."""
 
     hidden_size: int
     intermediate_size: int
@@ -393,6 +470,11 @@ class RoutedExpertsSpec:
     router: str = "sigmoid"
     renormalize: bool = False
     weight_on: str = "input"
+    choice_correction: bool = False
+    groups: Optional[tuple] = None
+    renorm_eps: float = 0.0
+    shared_intermediate: Optional[int] = None
+    shared_gate: bool = False
 
     def __post_init__(self):
         if min(self.hidden_size, self.intermediate_size, self.num_experts) < 1:
@@ -403,3 +485,15 @@ class RoutedExpertsSpec:
             raise ValueError(f"router {self.router!r}: expected 'sigmoid' or 'softmax'")
         if self.weight_on not in ("input", "output"):
             raise ValueError(f"weight_on {self.weight_on!r}: expected 'input' or 'output'")
+        if self.groups is not None:
+            if len(self.groups) != 3:
+                raise ValueError(f"groups is (count, kept, top), got {self.groups!r}")
+            count, kept, run_top = self.groups
+            if count < 1 or self.num_experts % count or not 1 <= kept <= count or run_top < 1:
+                raise ValueError(f"{self.num_experts} experts do not lie in {count} equal runs of which {kept} are kept")
+            if (self.num_experts // count) * kept < self.top_k:
+                raise ValueError(f"{kept} runs of {self.num_experts // count} experts cannot give {self.top_k} experts a token")
+        if self.shared_intermediate is not None and self.shared_intermediate < 1:
+            raise ValueError("the shared expert's inner width must be positive")
+        if self.shared_gate and self.shared_intermediate is None:
+            raise ValueError("a gate on the shared expert needs a shared expert")

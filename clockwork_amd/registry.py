@@ -41,6 +41,7 @@ _BUILTIN_ARCHITECTURES = {
     "Fuvavik": "clockwork_amd.models.fuvavik",
     "Pesorax": "clockwork_amd.models.pesorax",
     "Nenodra": "clockwork_amd.models.nenodra",
+    "Raranex": "clockwork_amd.models.raranex",
 }
 
 
@@ -107,11 +108,14 @@ _BUILTIN_PARTS = {
     "BranchRMSNormSpec": ("clockwork_amd.parts.norm", "BranchRMSNorm"),
     "GatedAttentionSpec": ("clockwork_amd.parts.gated_attention", "GatedAttention"),
     "RoutedExpertsSpec": ("clockwork_amd.parts.moe", "RoutedExperts"),
+    "ShiftedRecurrenceSpec": ("clockwork_amd.parts.linear_attention", "ShiftedRecurrence"),
+    "StreamReentrySpec": ("clockwork_amd.parts.embedding", "StreamReentry"),
 }
 _ARRANGEMENTS: dict[str, Callable[..., Any]] = {}
 _BUILTIN_ARRANGEMENTS = {"prenorm": ("clockwork_amd.parts.block", "PreNormBlock"),
                          "parallel": ("clockwork_amd.parts.block", "ParallelBlock"),
-                         "branchnorm": ("clockwork_amd.parts.block", "BranchNormBlock")}
+                         "branchnorm": ("clockwork_amd.parts.block", "BranchNormBlock"),
+                         "twonorm": ("clockwork_amd.parts.block", "TwoNormParallelBlock")}
 
 
 def register_part(spec_type: type, factory: Callable[[Any], Any]) -> None:
