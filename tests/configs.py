@@ -308,3 +308,119 @@ def random_nenodra_config(seed: int) -> dict:
             "residual_mult": rng.choice([0.3, 0.6, 1.0]), "logit_scale": rng.choice([0.25, 0.7, 2.0]),
             "norm": {"eps": rng.choice([1e-6, 1e-5])}, "layers": layers}
 
+
+
+# ------------------------------------------------------------------------------- Raranex
+def _raranex_window(heads, kv_heads, dim, vdim, scale, window, keep_first, base, rot_dims):
+    return {"heads": heads, "kv_heads": kv_heads, "dim": dim, "vdim": vdim, "scale": scale,
+            "mask": {"size": window, "keep_first": keep_first}, "rot": {"base": base, "dims": rot_dims}}
+
+
+def _raranex_pair(heads, kv_heads, dim, vdim, scale, softcap, coef, every, r_heads, r_dim, rank=None):
+    right = {"heads": r_heads, "dim": r_dim}
+    if rank is not None:
+        right["rank"] = rank
+    return {"left": {"heads": heads, "kv_heads": kv_heads, "dim": dim, "vdim": vdim, "scale": scale, "softcap": softcap,
+                     "q_temp": {"coef": coef, "every": every}}, "right": right}
+
+
+def _raranex_moe(ff, experts, top, groups=None, shared=None):
+    router = {"experts": experts, "top": top}
+    if groups is not None:
+        router["groups"] = {"count": groups[0], "keep": groups[1]}
+    mlp = {"kind": "moe", "expert": {"ff": ff}, "router": router}
+    if shared is not None:
+        mlp["shared"] = {"ff": shared}
+    return mlp
+
+
+# three layers of which the first two run twice: grouped heads with keys and values of unlike sizes,
+# a window of 9 that keeps 3 first tokens, a partial rotation, six experts in three runs of which two
+# are kept, a layer without a feed-forward, a decay projection of rank 6
+RARANEX_A = {
+    "architecture": "Raranex", "vocab": 211, "width": 96, "norm": {"eps": 1e-5},
+    "loop": {"start": 0, "stop": 2, "times": 2},
+    "layers": [
+        {"type": "parallel", "mixer": _raranex_pair(4, 2, 24, 16, 0.2, 8.0, 0.3, 7, 3, 16, rank=6),
+         "mlp": _raranex_moe(40, 6, 2, groups=(3, 2), shared=48)},
+        {"type": "attention", "mixer": _raranex_window(4, 4, 32, 24, 0.18, 9, 3, 100.0, 16), "mlp": None},
+        {"type": "attention", "mixer": _raranex_window(6, 2, 16, 40, 0.25, 33, 1, 10000.0, 16),
+         "mlp": _raranex_moe(24, 3, 3, shared=20)},
+    ],
+}
+# a width that is no multiple of 8, heads of 20 and 12 elements, a recurrence of one head whose size
+# is no multiple of 4, no loop, no expert runs, every expert chosen, no shared expert, a window of 1
+# (a token sees itself and the kept first ones) and a layer that only sees itself (nothing kept)
+RARANEX_B = {
+    "architecture": "Raranex", "vocab": 127, "width": 100, "norm": {"eps": 3e-4},
+    "layers": [
+        {"type": "attention", "mixer": _raranex_window(5, 5, 20, 12, 0.22, 1, 2, 50.0, 10), "mlp": _raranex_moe(36, 4, 4)},
+        {"type": "parallel", "mixer": _raranex_pair(3, 1, 40, 24, 0.16, 2.0, 1.5, 1, 1, 18), "mlp": _raranex_moe(50, 2, 1, shared=8)},
+        {"type": "attention", "mixer": _raranex_window(2, 1, 8, 32, 0.35, 1, 0, 10.0, 0), "mlp": None},
+    ],
+}
+# the whole model three times over, a window longer than any request of the tests, more first tokens
+# kept than the window holds, runs of one expert each, one expert a token, sizes of 1 and 2
+RARANEX_C = {
+    "architecture": "Raranex", "vocab": 64, "width": 48, "norm": {"eps": 1e-6},
+    "loop": {"start": 0, "stop": 2, "times": 3},
+    "layers": [
+        {"type": "attention", "mixer": _raranex_window(1, 1, 2, 1, 0.5, 300, 0, 4.0, 2), "mlp": _raranex_moe(1, 4, 1, groups=(4, 2), shared=1)},
+        {"type": "parallel", "mixer": _raranex_pair(1, 1, 32, 1, 0.18, 50.0, 0.0, 64, 2, 4, rank=1),
+         "mlp": _raranex_moe(16, 8, 3, groups=(2, 1), shared=24)},
+    ],
+}
+RARANEX_D = {
+    "architecture": "Raranex", "vocab": 90, "width": 64, "norm": {"eps": 1e-5},
+    "loop": {"start": 1, "stop": 2, "times": 2},
+    "layers": [
+        {"type": "attention", "mixer": _raranex_window(2, 2, 16, 16, 0.3, 4, 6, 1000.0, 16), "mlp": _raranex_moe(24, 4, 2, groups=(2, 1), shared=16)},
+        {"type": "parallel", "mixer": _raranex_pair(2, 2, 16, 8, 0.25, 5.0, 0.5, 3, 2, 8), "mlp": None},
+    ],
+}
+# name -> (config, weight seed, cache block size)
+RARANEX_CONFIGS = {"RA": (RARANEX_A, 51, 8), "RB": (RARANEX_B, 52, 16), "RC": (RARANEX_C, 53, 4), "RD": (RARANEX_D, 54, 8)}
+
+
+def random_raranex_config(seed: int) -> dict:
+    """A model of the design drawn at random: two to six layers that share nothing, a repeated run
+    anywhere among them (or none), head sizes that the matrix-core kernels take and ones they do
+    not, windows shorter and longer than a page with none to many first tokens kept, rotation of
+    all, a part and nothing, expert runs or none, a shared expert or none."""
+    import random
+
+    rng = random.Random(seed)
+    layers = []
+    for _ in range(rng.randint(2, 6)):
+        kv = rng.choice([1, 2, 4])
+        heads = kv * rng.choice([1, 2, 3, 4])
+        dim = rng.choice([16, 24, 32, 40, 48, 64, 80, 96, 128])
+        vdim = rng.choice([16, 24, 32, 48, 64, 96, 128])
+        scale = dim ** -0.5 * rng.choice([0.5, 1.0, 2.0])
+        experts = rng.choice([2, 4, 6, 8, 16])
+        top = rng.randint(1, min(4, experts))
+        groups = None
+        if rng.random() < 0.6:
+            count = rng.choice([c for c in (1, 2, 4, 8) if experts % c == 0])
+            keep = rng.randint(1, count)
+            if (experts // count) * keep >= top:
+                groups = (count, keep)
+        mlp = None if rng.random() < 0.15 else _raranex_moe(rng.choice([40, 64, 88, 128]), experts, top, groups,
+                                                               rng.choice([None, 32, 72, 128]))
+        if rng.random() < 0.5:
+            rot = rng.choice([dim, dim // 4 * 2, 16, 0, dim])
+            mixer = _raranex_window(heads, kv, dim, vdim, scale, rng.choice([1, 33, 64, 65, 100, 130, 200, 257]),
+                                    rng.choice([0, 1, 5, 64, 70, 150]), rng.choice([100.0, 10000.0, 5e5]), rot)
+            layers.append({"type": "attention", "mixer": mixer, "mlp": mlp})
+        else:
+            mixer = _raranex_pair(heads, kv, dim, vdim, scale, rng.choice([3.0, 20.0, 50.0]), rng.choice([0.0, 0.25, 1.0]),
+                                  rng.choice([1, 16, 64, 100]), rng.choice([1, 2, 4, 6]), rng.choice([8, 16, 20, 32, 64]),
+                                  rank=rng.choice([None, 4, 12, 32]))
+            layers.append({"type": "parallel", "mixer": mixer, "mlp": mlp})
+    cfg = {"architecture": "Raranex", "vocab": rng.choice([300, 500, 1000]), "width": rng.choice([128, 192, 320, 384]),
+           "norm": {"eps": rng.choice([1e-6, 1e-5])}, "layers": layers}
+    if rng.random() < 0.8:
+        start = rng.randint(0, len(layers) - 1)
+        cfg["loop"] = {"start": start, "stop": rng.randint(start + 1, len(layers)), "times": rng.randint(1, 3)}
+    return cfg
+
