@@ -2,7 +2,7 @@
 
     python bench.py [--gpus 1] [--steps K] [--warmup W] [--batch B] [--layers L] [--dtype bfloat16] [--shape 1.5b]
     python bench.py --workload mixed|arrivals|agent [--shape 7b] [--requests 64]
-    python bench.py --design fuvavik|pesorax|nenodra [--size s|m|l] [--layers L] [--batch B]
+    python bench.py --design fuvavik|pesorax|nenodra|raranex [--size s|m|l] [--layers L] [--batch B]
 
 Default workload: the layer sizes of Qwen2.5-1.5B with random weights (seed 2), bfloat16,
 8 requests that each hold a 2048-token prompt, context limit 4096, pages of 16 tokens. A
@@ -583,8 +583,41 @@ def nenodra_config(size: dict, layers: int, max_positions: int) -> dict:
             "layers": [{"type": kinds[i % 4][0], "mixer": kinds[i % 4][1], "mlp": kinds[i % 4][2]} for i in range(layers)]}
 
 
+# Layer sizes for ``--design raranex``: the same widths and head counts. Both attention mixers have
+# heads of the Qwen2 head's size; the window mixer sees half the prompt and the first 64 tokens; the
+# recurrence has as many heads of 64 x 64. Every layer's feed-forward is routed: eight experts of a
+# quarter of the Qwen2 layer's inner width in two runs of which one is kept, two experts a token,
+# and a shared expert of half that width (as many active parameters as the dense layer). Layers
+# alternate between the two kinds; the first two run twice behind a re-entry each (``layers`` counts
+# layer runs: the Qwen2 model beside it has that many layers).
+RARANEX_SIZES = {
+    "s": dict(width=896, heads=14, kv_heads=2, dim=64, vdim=64, head_dim=64, window=1024, keep_first=64, r_heads=14, r_dim=64,
+              rank=32, ff=4864, experts=8, top=2, layers=6),
+    "m": dict(width=1536, heads=12, kv_heads=2, dim=128, vdim=128, head_dim=128, window=1024, keep_first=64, r_heads=12, r_dim=64,
+              rank=64, ff=8960, experts=8, top=2, layers=6),
+    "l": dict(width=2048, heads=16, kv_heads=2, dim=128, vdim=128, head_dim=128, window=1024, keep_first=64, r_heads=16, r_dim=64,
+              rank=64, ff=11008, experts=8, top=2, layers=6),
+}
+
+
+def raranex_config(size: dict, layers: int, max_positions: int) -> dict:
+    routed = {"kind": "moe", "expert": {"ff": size["ff"] // 4}, "shared": {"ff": size["ff"] // 2},
+              "router": {"experts": size["experts"], "top": size["top"], "groups": {"count": 2, "keep": 1}}}
+    heads = {"heads": size["heads"], "kv_heads": size["kv_heads"], "dim": size["dim"], "vdim": size["vdim"], "scale": size["dim"] ** -0.5}
+    window = {"type": "attention", "mlp": routed,
+              "mixer": dict(heads, mask={"size": size["window"], "keep_first": size["keep_first"]}, rot={"base": 10000.0, "dims": 64})}
+    pair = {"type": "parallel", "mlp": routed,
+            "mixer": {"left": dict(heads, softcap=30.0, q_temp={"coef": 0.1, "every": 256}),
+                      "right": {"heads": size["r_heads"], "dim": size["r_dim"], "rank": size["rank"]}}}
+    # ``layers`` layer runs: the first two layers twice, the others once
+    distinct = max(2, layers - 2)
+    return {"architecture": "Raranex", "vocab": DESIGN_VOCAB, "width": size["width"], "norm": {"eps": 1e-5},
+            "loop": {"start": 0, "stop": 2, "times": 2 if layers >= 4 else 1},
+            "layers": [pair if i % 2 == 0 else window for i in range(distinct)]}
+
+
 DESIGNS = {"fuvavik": (FUVAVIK_SIZES, fuvavik_config), "pesorax": (PESORAX_SIZES, pesorax_config),
-           "nenodra": (NENODRA_SIZES, nenodra_config)}
+           "nenodra": (NENODRA_SIZES, nenodra_config), "raranex": (RARANEX_SIZES, raranex_config)}
 
 
 def qwen2_config_like(size: dict, layers: int, max_positions: int) -> dict:

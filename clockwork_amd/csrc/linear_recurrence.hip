@@ -5,7 +5,7 @@
 // with a weight shared by the heads and multiplied by silu(g_t).
 //
 // Variants (LinRecForm), for a recurrence of another family:
-//   decay_kind 1:  a_t = exp(-exp(z_t)) with z_t = A2 tanh(u_t) + b.
+//   decay_kind 1:  a_t = exp(-exp(z_t)) with z_t = A2 u_t + b;  2: the same with z_t = A2 tanh(u_t) + b.
 //   bonus [heads, dim]:  the output reads the state BEFORE the token joins it, and the token itself
 //                  through the bonus:  o_t = (S_(t-1) + diag(bonus) k_t v_t^T)^T q_t,  then
 //                  S_t = diag(a_t) S_(t-1) + k_t v_t^T.
@@ -24,7 +24,7 @@
 #define LR_TC 16  // tokens staged at a time
 
 struct LinRecForm {
-  int decay_kind;        // 0: sigmoid(z)^(1/tau); 1: exp(-exp(z)) with tanh on the decay input
+  int decay_kind;        // 0: sigmoid(z)^(1/tau); 1: exp(-exp(z)); 2: exp(-exp(z)) with tanh on the decay input
   const float* bonus;    // [heads, dim] or null
   int norm_w_stride;     // 0 or vdim
   const void* u;         // decay input rows, or null: columns u_off .. of proj
@@ -33,7 +33,7 @@ struct LinRecForm {
 };
 
 __device__ __forceinline__ float lr_decay(float z, int kind, float inv_tau) {
-  if (kind == 1) return expf(-expf(z));
+  if (kind >= 1) return expf(-expf(z));
   // log(sigmoid(z)) without cancellation, then the 1/tau-th power
   const float ls = z < 0.0f ? z - log1pf(expf(z)) : -log1pf(expf(-z));
   return expf(ls * inv_tau);
@@ -96,7 +96,7 @@ __global__ __launch_bounds__(256) void linear_recurrence_kernel(LinRecParams p, 
       float z = p.a2b ? p.a2b[h * D + d] : 0.0f;
       const T* w = a2 + (int64_t)(h * D + d) * p.rank;
       const T* u = f.u ? (const T*)f.u + (int64_t)(row0 + t0 + t) * f.u_stride : row + p.u_off;
-      if (f.decay_kind == 1) {
+      if (f.decay_kind == 2) {
         for (int c = 0; c < p.rank; ++c) z += cw_to_float(w[c]) * tanhf(cw_to_float(u[c]));
       } else {
         for (int c = 0; c < p.rank; ++c) z += cw_to_float(w[c]) * cw_to_float(u[c]);
@@ -183,7 +183,7 @@ CW_EXPORT int cw_linear_recurrence(int dtype, const void* proj, int64_t stride, 
   if (q_off % stride + heads * dim > stride || k_off % stride + heads * dim > stride || v_off % stride + heads * vdim > stride ||
       (!u && u_off + rank > stride) || (g_off >= 0 && g_off % stride + heads * vdim > stride))
     return CW_ERR_ARG;
-  if (decay_kind < 0 || decay_kind > 1 || (norm_w_stride != 0 && norm_w_stride != vdim) || (u && u_stride < rank) ||
+  if (decay_kind < 0 || decay_kind > 2 || (norm_w_stride != 0 && norm_w_stride != vdim) || (u && u_stride < rank) ||
       state_stride < (int64_t)heads * dim * vdim || state_stride > 0x7fffffff)
     return CW_ERR_ARG;
   if (!cw_linear_recurrence_supported(dim, vdim)) return CW_ERR_SIZE;
@@ -293,7 +293,9 @@ __global__ __launch_bounds__(256) void lrs_prepare_kernel(SegParams p) {
   const T* proj = (const T*)p.proj;
   const T* a2 = (const T*)p.a2;
   constexpr int N = LrVec<T>::N;
-  const bool vec = !p.form.u && p.rank % N == 0 && p.u_off % N == 0 && p.stride % N == 0 && !((uintptr_t)proj & 15) && !((uintptr_t)a2 & 15);
+  const bool vec = p.rank % N == 0 && !((uintptr_t)a2 & 15) &&
+                   (p.form.u ? p.form.u_stride % N == 0 && !((uintptr_t)p.form.u & 15)
+                             : p.u_off % N == 0 && p.stride % N == 0 && !((uintptr_t)proj & 15));
   for (int64_t idx = (int64_t)blockIdx.x * 256 + threadIdx.x; idx < n; idx += (int64_t)gridDim.x * 256) {
     const int64_t t = idx / HD;
     const int c = (int)(idx - t * HD);
@@ -301,7 +303,7 @@ __global__ __launch_bounds__(256) void lrs_prepare_kernel(SegParams p) {
     float z = p.a2b ? p.a2b[c] : 0.0f;
     const T* w = a2 + (int64_t)c * p.rank;
     const T* u = p.form.u ? (const T*)p.form.u + t * p.form.u_stride : row + p.u_off;
-    if (p.form.decay_kind == 1) {
+    if (p.form.decay_kind == 2) {
       for (int e = 0; e < p.rank; ++e) z += cw_to_float(w[e]) * tanhf(cw_to_float(u[e]));
     } else if (vec) {  // 16 bytes of the decay matrix's row and of the token's decay input at a time
       for (int e = 0; e < p.rank; e += N) {
@@ -492,7 +494,7 @@ CW_EXPORT int cw_linear_recurrence_segments(int dtype, const void* proj, int64_t
   if (q_off % stride + heads * dim > stride || k_off % stride + heads * dim > stride || v_off % stride + heads * vdim > stride ||
       (!u && u_off + rank > stride) || (g_off >= 0 && g_off % stride + heads * vdim > stride))
     return CW_ERR_ARG;
-  if (decay_kind < 0 || decay_kind > 1 || (norm_w_stride != 0 && norm_w_stride != vdim) || (u && u_stride < rank) ||
+  if (decay_kind < 0 || decay_kind > 2 || (norm_w_stride != 0 && norm_w_stride != vdim) || (u && u_stride < rank) ||
       state_stride < (int64_t)heads * dim * vdim || state_stride > 0x7fffffff)
     return CW_ERR_ARG;
   if (!cw_linear_recurrence_segments_supported(dim, vdim)) return CW_ERR_SIZE;

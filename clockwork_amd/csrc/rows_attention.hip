@@ -408,19 +408,26 @@ __global__ __launch_bounds__(256) void rows_mfma_kernel(const RowsAttnParams p, 
     for (int ks = 0; ks < D32; ++ks) qf[a][ks] = ra_load8(qrow + ks * 32);
   }
 
-  // this workgroup's run of the key chunks
-  const int n_chunks = (last - first) / RM_KT + 1;
+  // this workgroup's run of the key chunks. Behind a window that keeps a request's first
+  // positions visible, those of them that lie before the window's oldest key are chunks of their own,
+  // walked first; ``kept_end`` ends them.
+  const int kept_end = (p.mask_kind == RA_MASK_WINDOW && p.keep_first > 0) ? min(p.keep_first, first) : 0;
+  const int kept_chunks = (kept_end + RM_KT - 1) / RM_KT;
+  const int n_chunks = kept_chunks + (last - first) / RM_KT + 1;
   const int runs = gridDim.z;
   const int per_run = (n_chunks + runs - 1) / runs;
   const int c_begin = blockIdx.z * per_run, c_end = min(n_chunks, c_begin + per_run);
+  auto chunk_start = [&](int c) -> int { return c < kept_chunks ? c * RM_KT : first + (c - kept_chunks) * RM_KT; };
+  auto chunk_limit = [&](int c) -> int { return c < kept_chunks ? kept_end - 1 : last; };
 
   uint4 kreg[PFK], vreg[PFV];
   // A chunk's cache rows are looked up once, by 32 threads, and wait in LDS (two chunks' worth):
   // a lookup inside the fetch would put a load of the page table before every load of a row, and
   // since loads come home in order each row's load would wait for all the loads before it.
   __shared__ int chunk_rows[2][RM_KT];
-  auto row_of = [&](int j) -> int {
-    if (j > last) return -1;
+  auto row_of = [&](int c, int i) -> int {
+    const int j = chunk_start(c) + i;
+    if (j > chunk_limit(c)) return -1;
     const int b = j / p.block_size;
     const int page = b < p.table_width ? table[b] : -1;
     const int64_t row = (int64_t)page * p.block_size + j % p.block_size;
@@ -465,6 +472,8 @@ __global__ __launch_bounds__(256) void rows_mfma_kernel(const RowsAttnParams p, 
 
   constexpr float LOG2E = 1.4426950408889634f;
   const float scale2 = p.scale * LOG2E;
+  // the cap in units of log 2 as well: cap * tanh(score / cap) * log2(e)
+  const float cap2 = p.softcap * LOG2E, inv_cap2 = p.softcap > 0.0f ? 1.0f / cap2 : 0.0f;
   float m[UPW], l[UPW];
   ra_f32x4_t out[UPW][NT];
 #pragma unroll
@@ -485,13 +494,13 @@ __global__ __launch_bounds__(256) void rows_mfma_kernel(const RowsAttnParams p, 
   constexpr int VSTRIDE = ALIAS ? KROW : VROW;
 
   if (c_begin < c_end) {
-    if (tid < RM_KT) chunk_rows[0][tid] = row_of(first + c_begin * RM_KT + tid);
-    if (tid >= 64 && tid < 64 + RM_KT && c_begin + 1 < c_end) chunk_rows[1][tid - 64] = row_of(first + (c_begin + 1) * RM_KT + tid - 64);
+    if (tid < RM_KT) chunk_rows[0][tid] = row_of(c_begin, tid);
+    if (tid >= 64 && tid < 64 + RM_KT && c_begin + 1 < c_end) chunk_rows[1][tid - 64] = row_of(c_begin + 1, tid - 64);
     __syncthreads();
     fetch(chunk_rows[0]);
   }
   for (int c = c_begin; c < c_end; ++c) {
-    const int k0 = first + c * RM_KT;
+    const int k0 = chunk_start(c), limit = chunk_limit(c);
     __syncthreads();   // the tiles of the chunk before have been read; the rows of the next chunk are written
     store();
     if (c + 1 < c_end) fetch(chunk_rows[(c + 1 - c_begin) & 1]);
@@ -499,8 +508,9 @@ __global__ __launch_bounds__(256) void rows_mfma_kernel(const RowsAttnParams p, 
     // the rows of the chunk after the next: looked up now, written at the end of this round
     int later_row = -1;
     const bool looks_up = tid < RM_KT && c + 2 < c_end;
-    if (looks_up) later_row = row_of(k0 + 2 * RM_KT + tid);
-    const bool inside = nq == 16 && k0 + RM_KT - 1 <= pos0 && k0 >= lo_last;
+    if (looks_up) later_row = row_of(c + 2, tid);
+    // a chunk whose keys every query of the item sees needs no tests
+    const bool inside = nq == 16 && k0 + RM_KT - 1 <= min(pos0, limit) && (k0 >= lo_last || c < kept_chunks);
     ra_bf16x8_t pw[UPW];
 #pragma unroll
     for (int a = 0; a < UPW; ++a) {
@@ -520,7 +530,8 @@ __global__ __launch_bounds__(256) void rows_mfma_kernel(const RowsAttnParams p, 
       for (int u = 0; u < 8; ++u) {
         const int j = k0 + (u >> 2) * 16 + slot * 4 + (u & 3);
         float v = (u < 4 ? acc0[u & 3] : acc1[u & 3]) * scale2;
-        if (!inside) v = (l16 < nq && j <= pos && j >= lo) ? v : -INFINITY;
+        if (p.softcap > 0.0f) v = cap2 * tanhf(v * inv_cap2);
+        if (!inside) v = (l16 < nq && j <= min(pos, limit) && (j >= lo || j < p.keep_first)) ? v : -INFINITY;
         s[u] = v;
         top = fmaxf(top, v);
       }
@@ -705,13 +716,18 @@ __global__ __launch_bounds__(256) void rows_merge_kernel(const RowsAttnParams p,
 // How the matrix-core kernel cuts a geometry: value columns a workgroup takes (16 * nt), how many
 // workgroups share the columns, units a wave holds; 0 in *nt: not taken. Two maps: key rows of 64
 // or 128 elements a map, value rows of 64, 128 or 256 (the head norm needs all columns in one
-// workgroup). One map with the values inside the key row: key rows of 160, 320 or 576 elements,
+// workgroup). One map with values of their own: the same key and value sizes. One map with the values inside the key row: key rows of 160, 320 or 576 elements,
 // values their first 128, 256 or 512.
 static void ra_mfma_shape(int maps, int dim, int vdim, int alias, int* d32, int* nt, int* v_splits, int* upw) {
   *nt = 0; *v_splits = 1; *upw = maps == 2 ? 2 : 1; *d32 = dim / 32;
   if (dim % 32) return;
   if (maps == 2 && !alias) {
     if (*d32 != 2 && *d32 != 4) return;
+    if (vdim == 64) *nt = 4; else if (vdim == 128) *nt = 8; else if (vdim == 256) *nt = 16;
+  } else if (maps == 1 && !alias) {
+    // a wave holds two heads: eight heads of a key/value head's group a workgroup
+    if (*d32 != 2 && *d32 != 4) return;
+    *upw = 2;
     if (vdim == 64) *nt = 4; else if (vdim == 128) *nt = 8; else if (vdim == 256) *nt = 16;
   } else if (maps == 1 && alias) {
     if (*d32 == 5 && vdim == 128) *nt = 8;
@@ -748,10 +764,12 @@ CW_EXPORT int cw_rows_attention_mfma(const void* q, int64_t q_stride, int64_t q_
                                      const int* cu_q, const int* items, int n_items, const float* sink, const float* lambda,
                                      int heads, int kv_heads, int dim, int vdim, int maps, int block_size, int mask_kind,
                                      int mask_size, float scale, int head_norm, float norm_eps, float post_mult, int runs,
-                                     float* workspace, int64_t workspace_floats, hipStream_t stream) {
+                                     float* workspace, int64_t workspace_floats, int keep_first, float softcap,
+                                     hipStream_t stream) {
   if (n_items < 0 || !q || !out || !k_plane || !v_plane || !block_tables || !ctx_lens || !cu_q || !items) return CW_ERR_ARG;
   if (block_size <= 0 || table_width <= 0 || mask_kind < 0 || mask_kind > 2 || (mask_kind != 0 && mask_size < 1)) return CW_ERR_ARG;
   if ((maps == 2 && !lambda) || runs < 1 || runs > 64) return CW_ERR_ARG;
+  if (keep_first < 0 || (keep_first > 0 && mask_kind != RA_MASK_WINDOW) || softcap < 0.0f) return CW_ERR_ARG;
   const int alias = v_plane == k_plane;
   int d32, nt, vsp, upw;
   ra_mfma_shape(maps, dim, vdim, alias, &d32, &nt, &vsp, &upw);
@@ -772,7 +790,7 @@ CW_EXPORT int cw_rows_attention_mfma(const void* q, int64_t q_stride, int64_t q_
   p.ctx_lens = ctx_lens; p.cu_q = cu_q; p.items = items; p.sink = sink; p.lambda = lambda; p.heads = heads;
   p.kv_heads = kv_heads; p.dim = dim; p.vdim = vdim; p.maps = maps; p.heads_per_group = 0; p.tokens_per_item = 16;
   p.key_chunk = RM_KT; p.block_size = block_size; p.mask_kind = mask_kind; p.mask_size = mask_size; p.scale = scale;
-  p.head_norm = head_norm; p.norm_eps = norm_eps; p.post_mult = post_mult; p.keep_first = 0; p.softcap = 0.0f;
+  p.head_norm = head_norm; p.norm_eps = norm_eps; p.post_mult = post_mult; p.keep_first = keep_first; p.softcap = softcap;
   RowsMfmaExtra x;
   x.workspace = workspace; x.v_splits = vsp; x.heads_per_wg = maps == 2 ? 4 : 4 * upw;
   const int group = heads / kv_heads;
@@ -793,6 +811,13 @@ CW_EXPORT int cw_rows_attention_mfma(const void* q, int64_t q_stride, int64_t q_
     else if (nt == 4) CW_LAUNCH(4, 4, 2, 2, false);
     else if (nt == 8) CW_LAUNCH(4, 8, 2, 2, false);
     else CW_LAUNCH(4, 16, 2, 2, false);
+  } else if (!alias) {
+    if (d32 == 2 && nt == 4) CW_LAUNCH(2, 4, 2, 1, false);
+    else if (d32 == 2 && nt == 8) CW_LAUNCH(2, 8, 2, 1, false);
+    else if (d32 == 2) CW_LAUNCH(2, 16, 2, 1, false);
+    else if (nt == 4) CW_LAUNCH(4, 4, 2, 1, false);
+    else if (nt == 8) CW_LAUNCH(4, 8, 2, 1, false);
+    else CW_LAUNCH(4, 16, 2, 1, false);
   } else {
     if (d32 == 5) CW_LAUNCH(5, 8, 1, 1, true);
     else if (d32 == 10) CW_LAUNCH(10, 16, 1, 1, true);

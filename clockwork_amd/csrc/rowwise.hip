@@ -1029,6 +1029,24 @@ CW_EXPORT int cw_scale(float* x, int64_t n, float s, hipStream_t stream) {
   return cw_launch_status();
 }
 
+// ---------------------------------------------------------------- tanh, in place
+template <typename T>
+__global__ void tanh_kernel(T* __restrict__ x, int64_t n) {
+  for (int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; i < n; i += (int64_t)gridDim.x * blockDim.x)
+    x[i] = cw_from_float<T>(tanhf(cw_to_float(x[i])));
+}
+
+CW_EXPORT int cw_tanh(void* x, int dtype, int64_t n, hipStream_t stream) {
+  if (n < 0 || !x) return CW_ERR_ARG;
+  if (n == 0) return CW_OK;
+  int64_t blocks = (n + 255) / 256;
+  if (blocks > 65536) blocks = 65536;
+  if (dtype == CW_F32) hipLaunchKernelGGL(tanh_kernel<float>, dim3((unsigned)blocks), dim3(256), 0, stream, (float*)x, n);
+  else if (dtype == CW_BF16) hipLaunchKernelGGL(tanh_kernel<bf16_t>, dim3((unsigned)blocks), dim3(256), 0, stream, (bf16_t*)x, n);
+  else return CW_ERR_DTYPE;
+  return cw_launch_status();
+}
+
 // ---------------------------------------------------------------- mixes of a token with the one before it
 // out[s][t] = x[t] + (before[t] - x[t]) * mu[s], s < n_mix, float32 inside: ``before`` is the row
 // of the request's token one position earlier: the row above in x, or for the first token of a

@@ -136,6 +136,7 @@ def _declare(name: str, lib: ctypes.CDLL) -> None:
             "cw_branch_norm_add": [P, P, P, I, F, F, F, P, I, I, I, P],
             "cw_stream_norm": [P, P, I, F, F, P, I, P, I, I, P],
             "cw_headnorm_rope_store": [P, I, L, I, I, I, I, I, I, I, P, I, P, P, I, F, P, P, I, P, P, P, I, L, I, I, I, F, I, P],
+            "cw_tanh": [P, I, L, P],
             "cw_shift_mix": [P, I, P, I, I, P, L, L, I, P, P, P, I, P, L, I, P],
             "cw_stream_beside_input": [P, P, P, P, P, I, I, I, I, I, P],
             "cw_relu_squared": [P, I, L, P],
@@ -158,7 +159,7 @@ def _declare(name: str, lib: ctypes.CDLL) -> None:
             "cw_rows_mfma_grid_y": [I, I, I, I, I, I],
             "cw_rows_mfma_workspace_floats": [I, I, I, I, I, I, I, I],
             "cw_rows_attention_mfma": [P, L, L, P, L, L, P, P, I, I, L, P, I, P, P, P, I, P, P, I, I, I, I, I, I, I, I, F, I, F, F,
-                                       I, P, L, P],
+                                       I, P, L, I, F, P],
             "cw_rows_attention": [I, P, L, L, P, L, L, P, P, I, I, L, P, I, P, P, P, I, P, P, I, I, I, I, I, I, I, I, F, I, F, F,
                                   I, F, P],
         },
@@ -1443,7 +1444,7 @@ def linear_recurrence_supported(dim: int, vdim: int) -> bool:
     return bool(_load("linear_recurrence").cw_linear_recurrence_supported(dim, vdim))
 
 
-RECURRENCE_DECAYS = {"sigmoid_power": 0, "double_exp": 1}
+RECURRENCE_DECAYS = {"sigmoid_power": 0, "double_exp": 1, "double_exp_tanh": 2}
 
 
 def _recurrence_operands(proj, q_off, k_off, v_off, g_off, u_off, a2, a2_bias, norm_weight, state, heads, dim, vdim, decay, bonus,
@@ -1493,7 +1494,7 @@ def linear_recurrence(proj, q_off: int, k_off: int, v_off: int, g_off: int, u_of
 
     ``proj`` [planes, T, heads * dim]: q, k, v and the gate are planes, the offsets their numbers.
     ``decay_input`` [T, rank]: the decay's input as a tensor of its own. ``decay`` "double_exp":
-    a = exp(-exp(a2 tanh(input) + bias)). ``bonus`` float32 [heads, dim]: the output reads the
+    a = exp(-exp(a2 input + bias)); "double_exp_tanh": a = exp(-exp(a2 tanh(input) + bias)). ``bonus`` float32 [heads, dim]: the output reads the
     state before the token joins it and the token itself through the bonus,
     o = (S + diag(bonus) k v^T)^T q, then S <- diag(a) S + k v^T."""
     _gpu(proj, a2, a2_bias, norm_weight, state, state_slots, cu_q, bonus, decay_input)
@@ -1540,6 +1541,14 @@ def linear_recurrence_segments(proj, q_off: int, k_off: int, v_off: int, g_off: 
         int(seg_tokens), _ptr(req_first), _ptr(workspace), _ptr(out), n_requests, T, heads, dim, vdim, a2.shape[1], float(q_scale),
         1.0 / float(tau), float(eps), *tail, _stream()), "linear_recurrence_segments")
     return out
+
+
+def tanh_(x: torch.Tensor) -> torch.Tensor:
+    """x <- tanh(x), in place, float32 inside."""
+    _gpu(x)
+    _need(x.is_contiguous(), "tanh_ takes a dense tensor")
+    _check(_load("rowwise").cw_tanh(_ptr(x), dtype_code(x.dtype), x.numel(), _stream()), "tanh")
+    return x
 
 
 SHIFT_MIX_TOKENS = 16   # tokens of one request that a work item of ``shift_mix`` holds
@@ -1822,8 +1831,8 @@ ROWS_MFMA_TOKENS = 16   # tokens of one request that a work item of the matrix-c
 
 
 def rows_mfma_supported(dim: int, vdim: int, maps: int, dtype, alias: bool = False) -> bool:
-    """Does the matrix-core kernel take this geometry? bfloat16; two maps with key rows of 64 or
-    128 elements a map and value rows of 64, 128 or 256; or one map whose values lie inside the
+    """Does the matrix-core kernel take this geometry? bfloat16; one or two maps with key rows of 64
+    or 128 elements a map and value rows of 64, 128 or 256; or one map whose values lie inside the
     key row (``alias``): key rows of 160, 320 or 576 elements, values their first 128, 256 or 512."""
     return dtype == torch.bfloat16 and bool(_load("rows_attention").cw_rows_mfma_supported(maps, dim, vdim, int(alias)))
 
@@ -1920,7 +1929,6 @@ def rows_attention(q, q_strides, out, out_strides, k_plane, v_plane, block_table
     _need(keep_first >= 0 and (keep_first == 0 or mask == "window"), "first positions are kept visible behind a window only")
     _need(softcap >= 0.0, "a score cap is positive (0: none)")
     if mfma:
-        _need(keep_first == 0 and softcap == 0.0, "the matrix-core kernel has no kept first positions and no score cap")
         lib = _load("rows_attention")
         _need(rows_mfma_supported(dim, vdim, maps, q.dtype, alias), "the matrix-core kernel does not take this geometry")
         need = int(lib.cw_rows_mfma_workspace_floats(n_items, heads, kv_heads, maps, dim, vdim, int(alias), key_runs))
@@ -1930,7 +1938,7 @@ def rows_attention(q, q_strides, out, out_strides, k_plane, v_plane, block_table
             _ptr(block_tables), block_tables.shape[1], _ptr(ctx_lens), _ptr(cu_q), _ptr(items), n_items, _ptr(sink), _ptr(lam),
             heads, kv_heads, dim, vdim, maps, block_size, MASK_KINDS[mask], int(mask_size), float(scale),
             0 if head_norm_eps is None else 1, float(head_norm_eps or 0.0), float(post_mult), int(key_runs), _ptr(workspace), need,
-            _stream()), "rows_attention_mfma")
+            int(keep_first), float(softcap), _stream()), "rows_attention_mfma")
         return
     _check(_load("rows_attention").cw_rows_attention(
         dtype_code(q.dtype), _ptr(q), qs, qh, _ptr(out), os_, oh, _ptr(k_plane), _ptr(k_plane if alias else v_plane), k2.shape[1],

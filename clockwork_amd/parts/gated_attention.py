@@ -26,7 +26,7 @@ from clockwork_amd import ops
 from clockwork_amd.config.spec import PagedRowsSpec, ParamSpec
 from clockwork_amd.parts.attention import attention_plan
 from clockwork_amd.parts.base import EntryCache, Part
-from clockwork_amd.parts.sink_attention import query_runs
+from clockwork_amd.parts.sink_attention import longest_key_range, query_runs
 from clockwork_amd.parts.specs import GatedAttentionSpec, RopePairsSpec
 
 
@@ -93,9 +93,20 @@ class GatedAttention(Part):
                                 dtype=torch.float64)
             self.freq = freq.to(torch.float32).to(device)
         self.dtype = dtype
+        pad = (-self.in_width) % 8
+        if pad and dtype == torch.bfloat16:
+            # rows of the product that begin at multiples of 16 bytes (a few gate columns a head
+            # leave odd widths): the kernels behind it load 16 bytes a lane
+            self.in_weight = torch.cat([self.in_weight, self.in_weight.new_zeros((pad, s.hidden_size))])
+            if self.in_bias is not None:
+                self.in_bias = torch.cat([self.in_bias, self.in_bias.new_zeros(pad)])
         self.plain = self._plain_kernels(dtype) and ops.prefill_attention_supported(s.key_dim, dtype) \
             and ops.decode_attention_supported(s.key_dim, dtype)
-        if not self.plain:
+        # the matrix-core kernel for paged rows: bfloat16 heads of 64 or 128 elements with values of 64 to 256
+        self.mfma = not self.plain and ops.rows_mfma_supported(s.key_dim, s.value_dim, 1, dtype)
+        if self.mfma:
+            self.run = ops.ROWS_MFMA_TOKENS
+        elif not self.plain:
             if not ops.rows_attention_supported(s.num_heads, s.num_kv_heads, s.key_dim, s.value_dim, maps=1):
                 raise ValueError(f"attention with keys of {s.key_dim} and values of {s.value_dim} elements is beyond the "
                                  "attention kernel for paged rows (value_dim up to 512, tiles of 150 KB of LDS)")
@@ -105,7 +116,19 @@ class GatedAttention(Part):
         if self.plain:
             hd = self.spec.key_dim
             return attention_plan(ctx, self.spec.num_heads, self.spec.num_kv_heads, narrow_ok=ops.prefill_row_blocks_ok(hd, 2))
-        return query_runs(ctx, self.run)
+        if not self.mfma:
+            return (*query_runs(ctx, self.run), 1)
+        s = self.spec
+        key = ("gated attention", s.num_heads, s.num_kv_heads, s.key_dim, s.value_dim, s.window, s.keep_first)
+        plan = ctx.plans.get(key)
+        if plan is None:
+            items, n_items = query_runs(ctx, self.run)
+            # every item's keys are cut into runs where the step would leave most of the card idle
+            longest = longest_key_range(ctx, s.window) + (s.keep_first if s.window is not None else 0)
+            runs = ops.rows_mfma_key_runs(n_items, longest, s.num_heads, s.num_kv_heads, s.key_dim, s.value_dim, 1,
+                                          ctx.num_compute_units)
+            plan = ctx.plans[key] = (items, n_items, runs)
+        return plan
 
     def prepare(self, ctx) -> None:
         self._plan(ctx)
@@ -125,12 +148,12 @@ class GatedAttention(Part):
         if self.plain:
             self._attend_plain(proj, out, ctx, cache, k_plane, v_plane)
         else:
-            items, n_items = self._plan(ctx)
+            items, n_items, runs = self._plan(ctx)
             ops.rows_attention(proj, (proj.shape[1], s.key_dim), out, (out.shape[1], s.value_dim), k_plane, v_plane,
                                ctx.block_tables[cache.group], ctx.ctx_lens, ctx.cu_q, items, n_items, s.num_heads, s.num_kv_heads,
                                s.key_dim, s.value_dim, cache.block_size, s.scale, maps=1,
                                mask="window" if s.window is not None else "causal", mask_size=s.window or 0,
-                               keep_first=s.keep_first, softcap=s.softcap or 0.0)
+                               keep_first=s.keep_first, softcap=s.softcap or 0.0, mfma=self.mfma, key_runs=runs)
         if s.output_gate:
             bias_free = self.in_bias is None
             if not bias_free:

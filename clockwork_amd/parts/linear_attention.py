@@ -119,7 +119,7 @@ class ShiftedRecurrence(Part):
     waits in the request's state slot, and the portion's last row is left there); the products
     for r, k, v and the gate are one batched product over four planes, the decay's low-rank input
     a product of its own; the recurrence kernels of :class:`DecayedLinearAttention` walk the tokens
-    in their other form (the decay exp(-exp(.)) with tanh on its input, the output read from the
+    in their other form (the decay exp(-exp(.)) of the tanh of that input, the output read from the
     state before the token joins it, the token itself through the bonus), norm every head's output
     with the head's own weights and gate it; output product. Long portions are cut into segments
     that are walked side by side, as there. A request's slot is float32
@@ -192,11 +192,12 @@ class ShiftedRecurrence(Part):
         decay_input = ops.linear(mixes[4], self.decay_in, policy=policy)
         common = (planes, 0, 1, 2, 3, 0, self.decay_weight, self.decay_bias, self.norm_weight, state, ctx.state_slots, ctx.cu_q)
         sizes = (ctx.num_requests, s.num_heads, s.head_dim, s.head_dim, 1.0, 1.0, s.norm_eps)
-        form = dict(decay="double_exp", bonus=self.bonus, decay_input=decay_input)
         plan = self._segments(ctx)
         if plan is not None:
+            # a long portion: the tanh once an element, ahead of the kernel that makes every channel's decay from all of them
             seg_items, n_segments, first = plan
-            out = ops.linear_recurrence_segments(*common, seg_items, n_segments, SEGMENT_TOKENS, first, *sizes, **form)
+            out = ops.linear_recurrence_segments(*common, seg_items, n_segments, SEGMENT_TOKENS, first, *sizes, decay="double_exp",
+                                                 bonus=self.bonus, decay_input=ops.tanh_(decay_input))
         else:
-            out = ops.linear_recurrence(*common, *sizes, **form)
+            out = ops.linear_recurrence(*common, *sizes, decay="double_exp_tanh", bonus=self.bonus, decay_input=decay_input)
         return ops.linear(out, self.out_weight, policy=policy)
