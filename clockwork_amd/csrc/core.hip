@@ -50,7 +50,8 @@ template <typename T, typename WT, typename DT>
 __global__ void add_rmsnorm_kernel(float* __restrict__ resid, const T* __restrict__ delta0,
                                    const DT* __restrict__ delta, int parts,
                                    int64_t part_stride, const WT* __restrict__ weight, float eps,
-                                   T* __restrict__ out, const int* __restrict__ rows, int H) {
+                                   T* __restrict__ out, const int* __restrict__ rows, int H,
+                                   const WT* __restrict__ weight2, T* __restrict__ out2) {
   __shared__ float partial[4];
   const int i = blockIdx.x;
   const int t = rows ? rows[i] : i;
@@ -58,6 +59,7 @@ __global__ void add_rmsnorm_kernel(float* __restrict__ resid, const T* __restric
   const T* d0 = delta0 ? delta0 + (int64_t)t * H : nullptr;
   const DT* dl = delta ? delta + (int64_t)t * H : nullptr;
   T* o = out + (int64_t)i * H;
+  T* o2 = out2 ? out2 + (int64_t)i * H : nullptr;
   const bool write_back = rows == nullptr && (dl != nullptr || d0 != nullptr);
 
   float ss = 0.0f;
@@ -80,6 +82,7 @@ __global__ void add_rmsnorm_kernel(float* __restrict__ resid, const T* __restric
     if (dl && !write_back) v += delta_at(dl, part_stride, parts, j);
     const T n = cw_from_float<T>(v * inv);
     o[j] = cw_from_float<T>(cw_to_float(weight[j]) * cw_to_float(n));
+    if (o2) o2[j] = cw_from_float<T>(cw_to_float(weight2[j]) * cw_to_float(n));   // a second norm of the same row: its statistics are the first's
   }
 }
 
@@ -116,7 +119,8 @@ __global__ __launch_bounds__(256) void add_rmsnorm_vec_kernel(float* __restrict_
                                                               const DT* __restrict__ delta,
                                                               int parts, int64_t part_stride,
                                                               const WT* __restrict__ weight, float eps,
-                                                              T* __restrict__ out, const int* __restrict__ rows, int H) {
+                                                              T* __restrict__ out, const int* __restrict__ rows, int H,
+                                                              const WT* __restrict__ weight2, T* __restrict__ out2) {
   __shared__ float partial[4];
   const int i = blockIdx.x;
   const int t = rows ? rows[i] : i;
@@ -124,6 +128,7 @@ __global__ __launch_bounds__(256) void add_rmsnorm_vec_kernel(float* __restrict_
   const T* d0 = delta0 ? delta0 + (int64_t)t * H : nullptr;
   const DT* dl = delta ? delta + (int64_t)t * H : nullptr;
   T* o = out + (int64_t)i * H;
+  T* o2 = out2 ? out2 + (int64_t)i * H : nullptr;
   const bool write_back = rows == nullptr && (dl != nullptr || d0 != nullptr);
   const int n_chunks = H / 4;
   float v[KC][4], w[KC][4];
@@ -201,6 +206,13 @@ __global__ __launch_bounds__(256) void add_rmsnorm_vec_kernel(float* __restrict_
 #pragma unroll
       for (int e = 0; e < 4; ++e) r[e] = w[k][e] * cw_to_float(cw_from_float<T>(v[k][e] * inv));
       Chunk4<T>::store(o + ch * 4, r);
+      if (o2) {  // a second norm of the same row: its statistics are the first's
+        float w2[4];
+        Chunk4<WT>::load(weight2 + ch * 4, w2);
+#pragma unroll
+        for (int e = 0; e < 4; ++e) r[e] = w2[e] * cw_to_float(cw_from_float<T>(v[k][e] * inv));
+        Chunk4<T>::store(o2 + ch * 4, r);
+      }
     }
   }
 }
@@ -209,12 +221,13 @@ __global__ __launch_bounds__(256) void add_rmsnorm_vec_kernel(float* __restrict_
 // delta0: nullptr, or [T, H] in the activation type, added to the residual before delta.
 CW_EXPORT int cw_add_rmsnorm(float* resid, const void* delta0, const void* delta, int delta_parts, int T_rows,
                              const void* weight, int w_dtype, float eps, void* out, int dtype,
-                             const int* rows, int n, int H, hipStream_t stream) {
-  if (n < 0 || H <= 0 || delta_parts < 0 || delta_parts > 64) return CW_ERR_ARG;
+                             const int* rows, int n, int H, const void* weight2, void* out2, hipStream_t stream) {
+  if (n < 0 || H <= 0 || delta_parts < 0 || delta_parts > 64 || ((weight2 == nullptr) != (out2 == nullptr))) return CW_ERR_ARG;
   if (n == 0) return CW_OK;
   dim3 grid(n), block(256);
   const bool vec = (H % 4 == 0) && H <= 8192 && !((uintptr_t)resid & 15) && !((uintptr_t)out & 15) &&
-                   !((uintptr_t)weight & 15) && !((uintptr_t)delta & 15) && !((uintptr_t)delta0 & 15);
+                   !((uintptr_t)weight & 15) && !((uintptr_t)delta & 15) && !((uintptr_t)delta0 & 15) &&
+                   !((uintptr_t)weight2 & 15) && !((uintptr_t)out2 & 15);
   const int parts = delta_parts > 0 ? delta_parts : 1;
   const int64_t part_stride = (int64_t)T_rows * H;
 #define CW_LAUNCH(T, WT, DT)                                                                           \
@@ -222,15 +235,15 @@ CW_EXPORT int cw_add_rmsnorm(float* resid, const void* delta0, const void* delta
     if (vec && H <= 4096)                                                                              \
       hipLaunchKernelGGL((add_rmsnorm_vec_kernel<T, WT, DT, 4>), grid, block, 0, stream, resid,        \
                          (const T*)delta0, (const DT*)delta, parts, part_stride, (const WT*)weight, eps, \
-                         (T*)out, rows, H);                                                            \
+                         (T*)out, rows, H, (const WT*)weight2, (T*)out2);                                                            \
     else if (vec)                                                                                      \
       hipLaunchKernelGGL((add_rmsnorm_vec_kernel<T, WT, DT, 8>), grid, block, 0, stream, resid,        \
                          (const T*)delta0, (const DT*)delta, parts, part_stride, (const WT*)weight, eps, \
-                         (T*)out, rows, H);                                                            \
+                         (T*)out, rows, H, (const WT*)weight2, (T*)out2);                                                            \
     else                                                                                               \
       hipLaunchKernelGGL((add_rmsnorm_kernel<T, WT, DT>), grid, block, 0, stream, resid,               \
                          (const T*)delta0, (const DT*)delta, parts, part_stride, (const WT*)weight, eps, \
-                         (T*)out, rows, H);                                                            \
+                         (T*)out, rows, H, (const WT*)weight2, (T*)out2);                                                            \
   } while (0)
   if (delta_parts > 0) {
     if (dtype == CW_F32 && w_dtype == CW_F32) CW_LAUNCH(float, float, float);

@@ -50,6 +50,8 @@ struct MoeRouteOptions {
   int groups, groups_kept, group_top;   // groups <= 1: every expert can be chosen
   int extra;                // rows behind the router's E
   float* extra_out;         // [T, extra]
+  int renorm;               // the chosen scores are divided by their sum plus renorm_eps
+  float renorm_eps;
 };
 
 template <typename T>
@@ -172,16 +174,13 @@ __global__ __launch_bounds__(256) void moe_route_kernel(const T* __restrict__ x,
       if (found) z[at] = -3.4e38f;  // never chosen again
     }
   }
-}
-
-// the chosen scores of a token divided by their sum
-__global__ __launch_bounds__(64) void moe_renorm_kernel(float* __restrict__ score, int top, float eps) {
-  const int64_t t = blockIdx.x;
-  float sum = 0.0f;
-  for (int k = 0; k < top; ++k) sum += score[t * top + k];
-  sum += eps;
-  __syncthreads();
-  for (int k = threadIdx.x; k < top; k += 64) score[t * top + k] /= sum;
+  if (opt.renorm && lane == 0) {
+    // the lane that wrote the chosen scores divides them by their sum, added in the order of the choices
+    float sum = 0.0f;
+    for (int k = 0; k < top; ++k) sum += score[t * top + k];
+    sum += opt.renorm_eps;
+    for (int k = 0; k < top; ++k) score[t * top + k] /= sum;
+  }
 }
 
 // ---------------------------------------------------------------- 2. rows sorted by expert
@@ -652,7 +651,7 @@ CW_EXPORT int cw_moe_route(const void* x, const void* router, int dtype, int T, 
   if (groups > 1 && (E % groups || groups_kept < 1 || groups_kept > groups || group_top < 1 || group_top > MOE_MAX_GROUP_TOP ||
                      (E / groups) * groups_kept < top))
     return CW_ERR_ARG;
-  const MoeRouteOptions opt = {correction, groups, groups_kept, group_top, extra, extra_out};
+  const MoeRouteOptions opt = {correction, groups, groups_kept, group_top, extra, extra_out, renorm, renorm_eps};
   if (kind != MOE_ROUTER_SIGMOID && kind != MOE_ROUTER_SOFTMAX) return CW_ERR_ARG;
   if (E > MOE_MAX_EXPERTS) return CW_ERR_SIZE;
   if (T == 0) return CW_OK;
@@ -663,7 +662,6 @@ CW_EXPORT int cw_moe_route(const void* x, const void* router, int dtype, int T, 
     hipLaunchKernelGGL(moe_route_kernel<bf16_t>, dim3(T), dim3(256), 0, stream, (const bf16_t*)x, (const bf16_t*)router, H, E,
                        top, kind, choice, score, opt);
   else return CW_ERR_DTYPE;
-  if (renorm) hipLaunchKernelGGL(moe_renorm_kernel, dim3(T), dim3(64), 0, stream, score, top, renorm_eps);
   return cw_launch_status();
 }
 

@@ -12,6 +12,7 @@
 //             its own segment). With a window, the first ``keep_first`` positions of a request
 //             stay visible to every later token, at their true positions.
 //   * cap:    scores are squashed before the softmax: cap * tanh(scale * q . k / cap).
+//   * gate:   a head's output is multiplied by the logistic function of one number a token and head.
 //   * sink:   exp(sink[head]) joins the softmax denominator (no key, no value, not scaled).
 //   * norm:   the head's output is divided by its root mean square over vdim (eps inside the
 //             root) and multiplied by a constant.
@@ -51,7 +52,17 @@ struct RowsAttnParams {
   float norm_eps, post_mult;
   int keep_first;          // with a window: positions below this one are seen from anywhere later
   float softcap;           // > 0: score <- softcap * tanh(score / softcap)
+  const void* gate;        // or nullptr: head h of token t is multiplied by logistic(gate[t * gate_stride + gate_off + h])
+  int64_t gate_stride;
+  int gate_off;
 };
+
+template <typename T>
+__device__ __forceinline__ float ra_head_gate(const RowsAttnParams& p, int64_t token_row, int head) {
+  if (!p.gate) return 1.0f;
+  const float z = cw_to_float(((const T*)p.gate)[token_row * p.gate_stride + p.gate_off + head]);
+  return 1.0f / (1.0f + expf(-z));
+}
 
 __host__ __device__ inline int ra_key_stride(int maps, int dim) { return maps * dim + 1; }
 
@@ -231,6 +242,7 @@ __global__ __launch_bounds__(256) void rows_attention_kernel(const RowsAttnParam
     mult = p.post_mult / sqrtf(sq / (float)V + p.norm_eps);
   }
   if (live && m == 0) {
+    mult *= ra_head_gate<T>(p, trow, head);
     T* o = (T*)p.out + trow * p.out_stride + (int64_t)head * p.out_head_stride;
 #pragma unroll
     for (int i = 0; i < RA_MAXC; ++i) {
@@ -270,7 +282,8 @@ CW_EXPORT int cw_rows_attention(int dtype, const void* q, int64_t q_stride, int6
                                 const int* items, int n_items, const float* sink, const float* lambda, int heads,
                                 int kv_heads, int dim, int vdim, int maps, int block_size, int mask_kind,
                                 int mask_size, float scale, int head_norm, float norm_eps, float post_mult,
-                                int keep_first, float softcap, hipStream_t stream) {
+                                int keep_first, float softcap, const void* gate, int64_t gate_stride, int gate_off,
+                                hipStream_t stream) {
   if (n_items < 0 || !q || !out || !k_plane || !v_plane || !block_tables || !ctx_lens || !cu_q || !items)
     return CW_ERR_ARG;
   if (block_size <= 0 || table_width <= 0 || mask_kind < 0 || mask_kind > 2 || (mask_kind != 0 && mask_size < 1))
@@ -292,7 +305,8 @@ CW_EXPORT int cw_rows_attention(int dtype, const void* q, int64_t q_stride, int6
   p.kv_heads = kv_heads; p.dim = dim; p.vdim = vdim; p.maps = maps; p.heads_per_group = hc;
   p.tokens_per_item = RA_ROWS / (hc * maps); p.key_chunk = kc; p.block_size = block_size; p.mask_kind = mask_kind;
   p.mask_size = mask_size; p.scale = scale; p.head_norm = head_norm; p.norm_eps = norm_eps; p.post_mult = post_mult;
-  p.keep_first = keep_first; p.softcap = softcap;
+  p.keep_first = keep_first; p.softcap = softcap; p.gate = gate; p.gate_stride = gate_stride; p.gate_off = gate_off;
+  if (gate && (gate_stride < 1 || gate_off < 0)) return CW_ERR_ARG;
   const size_t smem = ra_lds_floats(maps, dim, vdim, kc, alias) * sizeof(float);
   const int group = heads / kv_heads;
   dim3 grid(n_items, kv_heads, (group + hc - 1) / hc), block(256);
@@ -622,6 +636,10 @@ __global__ __launch_bounds__(256) void rows_mfma_kernel(const RowsAttnParams p, 
       }
     }
     if (unit_ok[a]) {
+      if (p.gate) {
+#pragma unroll
+        for (int e = 0; e < 4; ++e) mult[e] *= ra_head_gate<bf16_t>(p, row0 + min(slot * 4 + e, nq - 1), unit_head[a]);
+      }
 #pragma unroll
       for (int nt = 0; nt < NT; ++nt)
 #pragma unroll
@@ -706,6 +724,7 @@ __global__ __launch_bounds__(256) void rows_merge_kernel(const RowsAttnParams p,
       sq = (scratch[0] + scratch[1]) + (scratch[2] + scratch[3]);
       mult = p.post_mult / sqrtf(sq / (float)p.vdim + p.norm_eps);
     }
+    mult *= ra_head_gate<bf16_t>(p, row0 + qi, head);
 #pragma unroll
     for (int i = 0; i < 2; ++i)
       if (tid + 256 * i < vw)
@@ -765,7 +784,7 @@ CW_EXPORT int cw_rows_attention_mfma(const void* q, int64_t q_stride, int64_t q_
                                      int heads, int kv_heads, int dim, int vdim, int maps, int block_size, int mask_kind,
                                      int mask_size, float scale, int head_norm, float norm_eps, float post_mult, int runs,
                                      float* workspace, int64_t workspace_floats, int keep_first, float softcap,
-                                     hipStream_t stream) {
+                                     const void* gate, int64_t gate_stride, int gate_off, hipStream_t stream) {
   if (n_items < 0 || !q || !out || !k_plane || !v_plane || !block_tables || !ctx_lens || !cu_q || !items) return CW_ERR_ARG;
   if (block_size <= 0 || table_width <= 0 || mask_kind < 0 || mask_kind > 2 || (mask_kind != 0 && mask_size < 1)) return CW_ERR_ARG;
   if ((maps == 2 && !lambda) || runs < 1 || runs > 64) return CW_ERR_ARG;
@@ -791,6 +810,8 @@ CW_EXPORT int cw_rows_attention_mfma(const void* q, int64_t q_stride, int64_t q_
   p.kv_heads = kv_heads; p.dim = dim; p.vdim = vdim; p.maps = maps; p.heads_per_group = 0; p.tokens_per_item = 16;
   p.key_chunk = RM_KT; p.block_size = block_size; p.mask_kind = mask_kind; p.mask_size = mask_size; p.scale = scale;
   p.head_norm = head_norm; p.norm_eps = norm_eps; p.post_mult = post_mult; p.keep_first = keep_first; p.softcap = softcap;
+  p.gate = gate; p.gate_stride = gate_stride; p.gate_off = gate_off;
+  if (gate && (gate_stride < 1 || gate_off < 0)) return CW_ERR_ARG;
   RowsMfmaExtra x;
   x.workspace = workspace; x.v_splits = vsp; x.heads_per_wg = maps == 2 ? 4 : 4 * upw;
   const int group = heads / kv_heads;

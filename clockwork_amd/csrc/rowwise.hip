@@ -1054,8 +1054,9 @@ CW_EXPORT int cw_tanh(void* x, int dtype, int64_t n, hipStream_t stream) {
 // state_stride floats; a request's first token ever finds zeros there, its slot being fresh).
 // items: (request, first token, tokens, 0), up to SHIFT_TOKENS tokens each. The workgroup of a
 // request's first item then leaves the portion's last row in the slot, for the next step: it alone
-// reads and writes the slot, in that order.
+// reads and writes the slot, in that order (a workgroup takes 256 columns of an item, a thread one).
 #define SHIFT_TOKENS 16
+#define SHIFT_MAX_MIXES 8
 template <typename T, typename WT>
 __global__ __launch_bounds__(256) void shift_mix_kernel(const T* __restrict__ x, const WT* __restrict__ mu, int n_mix,
                                                         float* __restrict__ state, int64_t state_stride, int64_t prev_off,
@@ -1070,32 +1071,34 @@ __global__ __launch_bounds__(256) void shift_mix_kernel(const T* __restrict__ x,
   const int slot = state_slots[req];
   const bool has_slot = slot >= 0 && slot < n_slots;
   float* kept = has_slot ? state + (int64_t)slot * state_stride + prev_off : nullptr;
+  // a thread owns one column of the item's tokens: what it reads of the slot it alone writes
+  const int j = blockIdx.y * 256 + threadIdx.x;
+  if (j >= W) return;
+  float m[SHIFT_MAX_MIXES];
+#pragma unroll
+  for (int s = 0; s < SHIFT_MAX_MIXES; ++s) m[s] = s < n_mix ? cw_to_float(mu[(int64_t)s * W + j]) : 0.0f;
+  float b = tok0 == 0 ? (kept ? kept[j] : 0.0f) : cw_to_float(x[((int64_t)row0 + tok0 - 1) * W + j]);
   for (int i = 0; i < ntok; ++i) {
     const int64_t row = (int64_t)row0 + tok0 + i;
-    const bool first = tok0 + i == 0;
-    for (int j = threadIdx.x; j < W; j += 256) {
-      const float v = cw_to_float(x[row * W + j]);
-      const float b = first ? (kept ? kept[j] : 0.0f) : cw_to_float(x[(row - 1) * W + j]);
-      for (int s = 0; s < n_mix; ++s)
-        out[((int64_t)s * n_tokens + row) * W + j] = cw_from_float<T>(v + (b - v) * cw_to_float(mu[(int64_t)s * W + j]));
-    }
+    const float v = cw_to_float(x[row * W + j]);
+#pragma unroll
+    for (int s = 0; s < SHIFT_MAX_MIXES; ++s)
+      if (s < n_mix) out[((int64_t)s * n_tokens + row) * W + j] = cw_from_float<T>(v + (b - v) * m[s]);
+    b = v;
   }
-  if (tok0 == 0 && kept) {
-    __syncthreads();  // every thread has read what the slot held
-    const int64_t last = (int64_t)row0 + q_len - 1;
-    for (int j = threadIdx.x; j < W; j += 256) kept[j] = cw_to_float(x[last * W + j]);
-  }
+  if (tok0 == 0 && kept) kept[j] = cw_to_float(x[((int64_t)row0 + q_len - 1) * W + j]);
 }
 
 CW_EXPORT int cw_shift_mix(const void* x, int dtype, const void* mu, int mu_dtype, int n_mix, float* state,
                            int64_t state_stride, int64_t prev_off, int n_slots, const int* state_slots, const int* cu_q,
                            const int* items, int n_items, void* out, int64_t n_tokens, int W, hipStream_t stream) {
   if (!x || !mu || !state || !state_slots || !cu_q || !items || !out) return CW_ERR_ARG;
-  if (n_mix < 1 || n_items < 0 || n_tokens < 0 || W < 1 || n_slots < 1 || prev_off < 0 || prev_off + W > state_stride)
+  if (n_mix < 1 || n_mix > SHIFT_MAX_MIXES || n_items < 0 || n_tokens < 0 || W < 1 || n_slots < 1 || prev_off < 0 ||
+      prev_off + W > state_stride)
     return CW_ERR_ARG;
   if (n_items == 0 || n_tokens == 0) return CW_OK;
 #define CW_LAUNCH(T_, WT_)                                                                                          \
-  hipLaunchKernelGGL((shift_mix_kernel<T_, WT_>), dim3(n_items), dim3(256), 0, stream, (const T_*)x, (const WT_*)mu, n_mix, \
+  hipLaunchKernelGGL((shift_mix_kernel<T_, WT_>), dim3(n_items, (W + 255) / 256), dim3(256), 0, stream, (const T_*)x, (const WT_*)mu, n_mix, \
                      state, state_stride, prev_off, n_slots, state_slots, cu_q, items, (T_*)out, n_tokens, W)
   if (dtype == CW_F32 && mu_dtype == CW_F32) CW_LAUNCH(float, float);
   else if (dtype == CW_BF16 && mu_dtype == CW_BF16) CW_LAUNCH(bf16_t, bf16_t);

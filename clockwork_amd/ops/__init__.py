@@ -94,7 +94,7 @@ def _declare(name: str, lib: ctypes.CDLL) -> None:
     sigs = {
         "core": {
             "cw_embedding": [P, I, P, P, I, I, I, P],
-            "cw_add_rmsnorm": [P, P, P, I, I, P, I, F, P, I, P, I, I, P],
+            "cw_add_rmsnorm": [P, P, P, I, I, P, I, F, P, I, P, I, I, P, P, P],
             "cw_rope_kv_write": [P, I, P, I, P, P, P, I, I, I, I, I, P, P, L, P],
             "cw_silu_mul": [P, P, I, I, I, P],
             "cw_copy_pages": [P, I, L, L, P, I, P],
@@ -159,9 +159,9 @@ def _declare(name: str, lib: ctypes.CDLL) -> None:
             "cw_rows_mfma_grid_y": [I, I, I, I, I, I],
             "cw_rows_mfma_workspace_floats": [I, I, I, I, I, I, I, I],
             "cw_rows_attention_mfma": [P, L, L, P, L, L, P, P, I, I, L, P, I, P, P, P, I, P, P, I, I, I, I, I, I, I, I, F, I, F, F,
-                                       I, P, L, I, F, P],
+                                       I, P, L, I, F, P, L, I, P],
             "cw_rows_attention": [I, P, L, L, P, L, L, P, P, I, I, L, P, I, P, P, P, I, P, P, I, I, I, I, I, I, I, I, F, I, F, F,
-                                  I, F, P],
+                                  I, F, P, L, I, P],
         },
         "sink_attention": {
             "cw_sink_attention_max_bq": [I, I, I, I],
@@ -323,11 +323,13 @@ class LazyAddNorm:
         return add_rmsnorm(self.resid, self.delta, self.weight, self.eps, out, write_back=False)
 
 
-def add_rmsnorm(resid, delta, weight, eps: float, out, rows=None, write_back: bool = True) -> torch.Tensor:
+def add_rmsnorm(resid, delta, weight, eps: float, out, rows=None, write_back: bool = True, weight2=None, out2=None) -> torch.Tensor:
     """resid += delta (when given), out = rmsnorm(resid) * weight; with ``rows`` only those rows
     are normed into out[i] and resid is left alone, as it is with ``write_back`` off. resid
     float32 [T, H]; delta/out in the activation type, or delta a :class:`PartialSums` of that
-    shape, or a :class:`PendingPair` (both are added, ``first`` first)."""
+    shape, or a :class:`PendingPair` (both are added, ``first`` first). ``weight2`` / ``out2``: a
+    second norm of the same rows with weights of its own (the same eps, so the same statistics),
+    written beside the first by the same kernel."""
     delta0 = None
     if isinstance(delta, PendingPair):
         delta0, delta = delta.first, delta.second
@@ -351,6 +353,12 @@ def add_rmsnorm(resid, delta, weight, eps: float, out, rows=None, write_back: bo
         raise KernelError(f"out must be [{n}, {H}]")
     if not (weight.numel() == H):
         raise KernelError("norm weight has the wrong size")
+    if (weight2 is None) != (out2 is None):
+        raise KernelError("a second norm needs its weights and its output")
+    if weight2 is not None:
+        _gpu(weight2, out2)
+        if not (weight2.numel() == H and weight2.dtype == weight.dtype and tuple(out2.shape) == (n, H) and out2.dtype == out.dtype):
+            raise KernelError("the second norm's weights and output must match the first's")
     if parts:
         if not (tuple(delta.shape) == (parts, T, H) and delta.dtype == torch.float32):
             raise KernelError("partial sums must be float32 [parts, T, H]")
@@ -360,7 +368,7 @@ def add_rmsnorm(resid, delta, weight, eps: float, out, rows=None, write_back: bo
     _check(
         _load("core").cw_add_rmsnorm(
             _ptr(resid), _ptr(delta0), _ptr(delta), parts, T, _ptr(weight), dtype_code(weight.dtype), float(eps), _ptr(out),
-            dtype_code(out.dtype), _ptr(rows), n, H, _stream()),
+            dtype_code(out.dtype), _ptr(rows), n, H, _ptr(weight2), _ptr(out2), _stream()),
         "add_rmsnorm",
     )
     return out
@@ -1878,7 +1886,7 @@ def rows_attention(q, q_strides, out, out_strides, k_plane, v_plane, block_table
                    heads: int, kv_heads: int, dim: int, vdim: int, block_size: int, scale: float, maps: int = 1,
                    mask: str = "causal", mask_size: int = 0, sink=None, lam=None, head_norm_eps=None,
                    post_mult: float = 1.0, mfma: bool = False, key_runs: int = 1, keep_first: int = 0,
-                   softcap: float = 0.0) -> None:
+                   softcap: float = 0.0, head_gate=None) -> None:
     """Softmax attention of the step's queries over paged rows. Query (t, head, map, d) lies at
     ``q.flatten()[t * q_strides[0] + head * q_strides[1] + map * dim + d]``, output (t, head, c) at
     ``out.flatten()[t * out_strides[0] + head * out_strides[1] + c]`` (token-major or head-major
@@ -1889,7 +1897,8 @@ def rows_attention(q, q_strides, out, out_strides, k_plane, v_plane, block_table
     tokens of the token's segment of ``mask_size`` positions, segments counted from position 0).
     ``keep_first`` n (with a window): the request's first n positions stay visible to every later
     token. ``softcap`` c > 0: scores are squashed, c * tanh(scale * q . k / c), before the softmax.
-    ``sink`` float32 [heads]: exp(sink) joins the denominator. ``maps`` 2: the head's output is
+    ``head_gate`` (z, offset): head h of token t is multiplied by logistic(z[t, offset + h]), z [T, width]
+    in the queries' type. ``sink`` float32 [heads]: exp(sink) joins the denominator. ``maps`` 2: the head's output is
     map 0 minus ``lam`` (one float32 element) times map 1. ``head_norm_eps`` not None: the head's
     output is divided by its root mean square and multiplied by ``post_mult``. ``items`` int32
     [n_items, 4]: (request, first token, tokens, 0) with at most
@@ -1928,6 +1937,13 @@ def rows_attention(q, q_strides, out, out_strides, k_plane, v_plane, block_table
     _need(mask in MASK_KINDS and (mask == "causal" or mask_size >= 1), f"mask {mask!r} of size {mask_size}")
     _need(keep_first >= 0 and (keep_first == 0 or mask == "window"), "first positions are kept visible behind a window only")
     _need(softcap >= 0.0, "a score cap is positive (0: none)")
+    gate, gate_stride, gate_off = None, 0, 0
+    if head_gate is not None:
+        gate, gate_off = head_gate
+        _gpu(gate)
+        _need(gate.dim() == 2 and gate.dtype == q.dtype and gate.shape[0] >= tokens and gate.is_contiguous()
+              and 0 <= gate_off and gate_off + heads <= gate.shape[1], "the gates must be [T, width] with a column a head")
+        gate_stride = gate.shape[1]
     if mfma:
         lib = _load("rows_attention")
         _need(rows_mfma_supported(dim, vdim, maps, q.dtype, alias), "the matrix-core kernel does not take this geometry")
@@ -1938,14 +1954,14 @@ def rows_attention(q, q_strides, out, out_strides, k_plane, v_plane, block_table
             _ptr(block_tables), block_tables.shape[1], _ptr(ctx_lens), _ptr(cu_q), _ptr(items), n_items, _ptr(sink), _ptr(lam),
             heads, kv_heads, dim, vdim, maps, block_size, MASK_KINDS[mask], int(mask_size), float(scale),
             0 if head_norm_eps is None else 1, float(head_norm_eps or 0.0), float(post_mult), int(key_runs), _ptr(workspace), need,
-            int(keep_first), float(softcap), _stream()), "rows_attention_mfma")
+            int(keep_first), float(softcap), _ptr(gate), int(gate_stride), int(gate_off), _stream()), "rows_attention_mfma")
         return
     _check(_load("rows_attention").cw_rows_attention(
         dtype_code(q.dtype), _ptr(q), qs, qh, _ptr(out), os_, oh, _ptr(k_plane), _ptr(k_plane if alias else v_plane), k2.shape[1],
         v_row, rows, _ptr(block_tables), block_tables.shape[1], _ptr(ctx_lens), _ptr(cu_q), _ptr(items), n_items, _ptr(sink),
         _ptr(lam), heads, kv_heads, dim, vdim, maps, block_size, MASK_KINDS[mask], int(mask_size), float(scale),
         0 if head_norm_eps is None else 1, float(head_norm_eps or 0.0), float(post_mult), int(keep_first), float(softcap),
-        _stream()), "rows_attention")
+        _ptr(gate), int(gate_stride), int(gate_off), _stream()), "rows_attention")
 
 
 # ---------------------------------------------------------------------------------------------

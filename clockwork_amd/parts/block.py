@@ -148,7 +148,7 @@ class TwoNormParallelBlock:
 
     def forward(self, resid, delta, ctx, cache):
         both = getattr(self.mixer_norm, "forward_pair", None)
-        if self.feed_forward is not None and both is not None:
+        if self.feed_forward is not None and both is not None and type(self.ffn_norm) is type(self.mixer_norm):
             x, y = both(resid, delta, self.ffn_norm)   # one kernel: the two norms share the row's statistics
         else:
             x = self.mixer_norm.forward(resid, delta)

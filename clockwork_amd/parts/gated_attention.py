@@ -103,8 +103,10 @@ class GatedAttention(Part):
         self.plain = self._plain_kernels(dtype) and ops.prefill_attention_supported(s.key_dim, dtype) \
             and ops.decode_attention_supported(s.key_dim, dtype)
         # the matrix-core kernel for paged rows: bfloat16 heads of 64 or 128 elements with values of 64 to 256
-        self.mfma = not self.plain and ops.rows_mfma_supported(s.key_dim, s.value_dim, 1, dtype)
-        if self.mfma:
+        self.rows_mfma = not self.plain and ops.rows_mfma_supported(s.key_dim, s.value_dim, 1, dtype)
+        # a gate a head without a bias is applied where the attention kernel stores a head
+        self._gate_inside = s.output_gate and s.gate_per_head and self.in_bias is None
+        if self.rows_mfma:
             self.run = ops.ROWS_MFMA_TOKENS
         elif not self.plain:
             if not ops.rows_attention_supported(s.num_heads, s.num_kv_heads, s.key_dim, s.value_dim, maps=1):
@@ -116,7 +118,7 @@ class GatedAttention(Part):
         if self.plain:
             hd = self.spec.key_dim
             return attention_plan(ctx, self.spec.num_heads, self.spec.num_kv_heads, narrow_ok=ops.prefill_row_blocks_ok(hd, 2))
-        if not self.mfma:
+        if not self.rows_mfma:
             return (*query_runs(ctx, self.run), 1)
         s = self.spec
         key = ("gated attention", s.num_heads, s.num_kv_heads, s.key_dim, s.value_dim, s.window, s.keep_first)
@@ -153,8 +155,9 @@ class GatedAttention(Part):
                                ctx.block_tables[cache.group], ctx.ctx_lens, ctx.cu_q, items, n_items, s.num_heads, s.num_kv_heads,
                                s.key_dim, s.value_dim, cache.block_size, s.scale, maps=1,
                                mask="window" if s.window is not None else "causal", mask_size=s.window or 0,
-                               keep_first=s.keep_first, softcap=s.softcap or 0.0, mfma=self.mfma, key_runs=runs)
-        if s.output_gate:
+                               keep_first=s.keep_first, softcap=s.softcap or 0.0, mfma=self.rows_mfma, key_runs=runs,
+                               head_gate=(proj, self.g_off) if self._gate_inside else None)
+        if s.output_gate and not (self._gate_inside and not self.plain):
             bias_free = self.in_bias is None
             if not bias_free:
                 raise NotImplementedError("an output gate with a bias")

@@ -29,6 +29,17 @@ class RMSNorm(Part):
         out = torch.empty((n, self.spec.size), dtype=self.dtype, device=resid.device)
         return ops.add_rmsnorm(resid, delta, self.weight, self.spec.eps, out, rows)
 
+    def forward_pair(self, resid: torch.Tensor, delta, other: "RMSNorm"):
+        """(this norm, ``other``'s norm) of resid + delta in one kernel: two norms of the same rows
+        share the statistics when their eps agree; else two kernels."""
+        if other.spec.eps != self.spec.eps or other.spec.size != self.spec.size or other.weight.dtype != self.weight.dtype:
+            return self.forward(resid, delta), other.forward(resid, None)
+        shape = (resid.shape[0], self.spec.size)
+        out = torch.empty(shape, dtype=self.dtype, device=resid.device)
+        out2 = torch.empty(shape, dtype=self.dtype, device=resid.device)
+        ops.add_rmsnorm(resid, delta, self.weight, self.spec.eps, out, weight2=other.weight, out2=out2)
+        return out, out2
+
     def lazy(self, resid: torch.Tensor, delta) -> "ops.LazyAddNorm":
         """The norm of resid + delta for a consumer that computes it inside its own kernel; the
         residual is not updated, so ``delta`` has to reach the next norm as well."""
