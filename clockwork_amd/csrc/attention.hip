@@ -37,6 +37,7 @@ struct AttnParams {
   int n_splits;
   int window;             // 0: none
   float scale;
+  float softcap;          // > 0: score <- softcap * tanh(scale * q . k / softcap) (the matrix-core kernels)
   float* part_o;          // [n_items, nkv * n_chunks, n_splits, ROWS, HD] unnormalised outputs
   float* part_ml;         // [n_items, nkv * n_chunks, n_splits, ROWS, 2] running max, sum
   const void* zeros;      // at least HD zero elements: what a masked key or value row is loaded from
@@ -396,7 +397,7 @@ CW_EXPORT int cw_attention(int rows, int dtype, const void* q, int64_t q_stride,
   p.k_cache = k_cache; p.v_cache = v_cache; p.block_tables = block_tables;
   p.table_stride = table_stride; p.ctx_lens = ctx_lens; p.cu_q = cu_q; p.items = items;
   p.nh = nh; p.nkv = nkv; p.block_size = block_size; p.bs_shift = cw_log2_or_minus1(block_size); p.gh = gh;
-  p.n_chunks = (group + gh - 1) / gh; p.n_splits = n_splits; p.window = window; p.scale = scale;
+  p.n_chunks = (group + gh - 1) / gh; p.n_splits = n_splits; p.window = window; p.scale = scale; p.softcap = 0.0f;
   if ((int64_t)nkv * p.n_chunks > 65535) return CW_ERR_SIZE;
   const int64_t need = cw_attention_workspace_floats(rows, n_items, nkv, p.n_chunks, n_splits);
   if (need > 0 && (workspace == nullptr || workspace_floats < need)) return CW_ERR_ARG;
@@ -550,7 +551,9 @@ __global__ __launch_bounds__(256) void attn_decode_bf16_kernel(AttnParams p) {
 #pragma unroll
       for (int i = 0; i < 4; ++i) {
         const int kp = kv0 + kb * 16 + 4 * s + i;
-        const float v = (kp >= lo && kp <= pos) ? sc[i] * p.scale : -INFINITY;
+        float v = sc[i] * p.scale;
+        if (p.softcap > 0.0f) v = p.softcap * tanhf(v / p.softcap);
+        v = (kp >= lo && kp <= pos) ? v : -INFINITY;
         sv[kb * 4 + i] = v;
         tmax = fmaxf(tmax, v);
       }
@@ -775,7 +778,7 @@ CW_EXPORT int cw_attention_decode_bf16(const void* q, int64_t q_stride, void* ou
                                        const int* items, int n_items, int nh, int nkv, int block_size,
                                        int n_splits, int window, float scale, float* workspace,
                                        int64_t workspace_floats, const void* zeros, int identity,
-                                       int split_keys, int max_ctx, hipStream_t stream) {
+                                       int split_keys, int max_ctx, float softcap, hipStream_t stream) {
 #if CW_HAS_DECODE
   if (n_items < 0 || nh <= 0 || nkv <= 0 || nh % nkv != 0 || block_size <= 0 || table_stride <= 0)
     return CW_ERR_ARG;
@@ -795,7 +798,7 @@ CW_EXPORT int cw_attention_decode_bf16(const void* q, int64_t q_stride, void* ou
   p.nh = nh; p.nkv = nkv; p.block_size = block_size; p.bs_shift = cw_log2_or_minus1(block_size);
   p.identity = identity ? 1 : 0; p.split_keys = split_keys;
   p.gh = cw_attention_decode_gh(group);
-  p.n_chunks = (group + p.gh - 1) / p.gh; p.n_splits = n_splits; p.window = window; p.scale = scale;
+  p.n_chunks = (group + p.gh - 1) / p.gh; p.n_splits = n_splits; p.window = window; p.scale = scale; p.softcap = softcap;
   if ((int64_t)nkv * p.n_chunks * p.gh > 65535) return CW_ERR_SIZE;
   const int64_t need = cw_attention_decode_workspace_floats(n_items, nh, nkv, n_splits);
   if (need > 0 && (workspace == nullptr || workspace_floats < need)) return CW_ERR_ARG;
@@ -1028,6 +1031,16 @@ __global__ __launch_bounds__((PrefillTile<HD, RB>::NT), (HD <= 128 ? 2 : 1)) voi
           for (int j = 0; j < NF; ++j)
             sc[kb][b] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(kf[j], qf[b][j], sc[kb][b], 0, 0, 0);
         }
+      }
+      if (p.softcap > 0.0f) {
+        // capped scores, kept in units of the raw score: s <- (cap / scale) * tanh(s * scale / cap)
+        const float up = p.softcap / p.scale, down = p.scale / p.softcap;
+#pragma unroll
+        for (int kb = 0; kb < NKB; ++kb)
+#pragma unroll
+          for (int b = 0; b < 2; ++b)
+#pragma unroll
+            for (int i = 0; i < 4; ++i) sc[kb][b][i] = up * tanhf(sc[kb][b][i] * down);
       }
       // ---- softmax per row; P^T packed as the B operand of the output product.
       // A tile needs the position tests only if some row of the wave masks some key of it.
@@ -1367,7 +1380,7 @@ CW_EXPORT int cw_attention_prefill_bf16(const void* q, int64_t q_stride, void* o
                                         const int* items, int n_items, int nh, int nkv, int block_size,
                                         int window, float scale, const void* zeros, int row_blocks,
                                         int with_parts, float* workspace, int64_t workspace_floats,
-                                        hipStream_t stream) {
+                                        float softcap, hipStream_t stream) {
 #if CW_HAS_PREFILL
   if (zeros == nullptr || ((uintptr_t)zeros & 15)) return CW_ERR_ARG;
   if (n_items < 0 || nh <= 0 || nkv <= 0 || nh % nkv != 0 || block_size <= 0 || table_stride <= 0 || window < 0)
@@ -1383,7 +1396,7 @@ CW_EXPORT int cw_attention_prefill_bf16(const void* q, int64_t q_stride, void* o
   p.k_cache = k_cache; p.v_cache = v_cache; p.block_tables = block_tables;
   p.table_stride = table_stride; p.ctx_lens = ctx_lens; p.cu_q = cu_q; p.items = items;
   p.nh = nh; p.nkv = nkv; p.block_size = block_size; p.bs_shift = cw_log2_or_minus1(block_size); p.gh = group < 32 ? group : 32;
-  p.n_chunks = (group + p.gh - 1) / p.gh; p.n_splits = 1; p.window = window; p.scale = scale;
+  p.n_chunks = (group + p.gh - 1) / p.gh; p.n_splits = 1; p.window = window; p.scale = scale; p.softcap = softcap;
   p.part_o = nullptr; p.part_ml = nullptr; p.zeros = zeros;
   if ((int64_t)nkv * p.n_chunks > 65535) return CW_ERR_SIZE;
   if (with_parts) {

@@ -193,14 +193,14 @@ def _declare(name: str, lib: ctypes.CDLL) -> None:
             "cw_attention_workspace_floats": [I, I, I, I, I],
             "cw_attention": [I, I, P, L, P, L, P, P, P, I, P, P, P, I, I, I, I, I, I, I, F, P, L, P],
             "cw_attention_prefill_supported": [],
-            "cw_attention_prefill_bf16": [P, L, P, L, P, P, P, I, P, P, P, I, I, I, I, I, F, P, I, I, P, L, P],
+            "cw_attention_prefill_bf16": [P, L, P, L, P, P, P, I, P, P, P, I, I, I, I, I, F, P, I, I, P, L, F, P],
             "cw_attention_prefill_workspace_floats": [I, I, I, I],
             "cw_attention_prefill_row_blocks_ok": [I],
             "cw_attention_decode_supported": [],
             "cw_attention_decode_gh": [I],
             "cw_attention_decode_max_splits": [],
             "cw_attention_decode_workspace_floats": [I, I, I, I],
-            "cw_attention_decode_bf16": [P, L, P, L, P, P, P, I, P, P, P, I, I, I, I, I, I, F, P, L, P, I, I, I, P],
+            "cw_attention_decode_bf16": [P, L, P, L, P, P, P, I, P, P, P, I, I, I, I, I, I, F, P, L, P, I, I, I, F, P],
         },
     }[name]
     for fn, argtypes in sigs.items():
@@ -1050,8 +1050,9 @@ def prefill_attention_supported(hd: int, dtype: torch.dtype) -> bool:
 
 def attention_prefill(q, q_stride: int, out, k_cache, v_cache, block_tables, ctx_lens, cu_q, items, n_items: int,
                       nh: int, nkv: int, hd: int, block_size: int, window: int, scale: float,
-                      n_tokens: int, n_requests: int, row_blocks: int = 4, workspace=None) -> None:
-    """Portions of prompts through the bfloat16 matrix-core kernel; an item holds at most
+                      n_tokens: int, n_requests: int, row_blocks: int = 4, workspace=None, softcap: float = 0.0) -> None:
+    """Portions of prompts through the bfloat16 matrix-core kernel (``softcap`` c > 0: scores are
+    squashed, c * tanh(scale * q . k / c), before the softmax); an item holds at most
     ``prefill_tokens_per_item(nh // nkv, row_blocks)`` tokens. ``row_blocks`` 2 instead of 4: smaller
     workgroups for launches with few items (head sizes up to 128). Other arguments as for ``attention``.
     An item's fourth field is ``part | parts << 8``: with parts > 1 the item stands that many times
@@ -1086,7 +1087,7 @@ def attention_prefill(q, q_stride: int, out, k_cache, v_cache, block_tables, ctx
             q.data_ptr(), int(q_stride), _ptr(out), out.shape[1], _ptr(k_cache), _ptr(v_cache), _ptr(block_tables),
             block_tables.shape[1], _ptr(ctx_lens), _ptr(cu_q), _ptr(items), n_items, nh, nkv, block_size,
             window, float(scale), _zero_row(out.device), int(row_blocks), int(workspace is not None), _ptr(workspace),
-            ws_floats, _stream()),
+            ws_floats, float(softcap), _stream()),
         "attention_prefill_bf16",
     )
 
@@ -1120,8 +1121,9 @@ def decode_attention_workspace_floats(hd: int, n_items: int, nh: int, nkv: int, 
 def attention_decode(q, q_stride: int, out, k_cache, v_cache, block_tables, ctx_lens, cu_q, items, n_items: int,
                      nh: int, nkv: int, hd: int, block_size: int, n_splits: int, window: int, scale: float,
                      n_tokens: int, n_requests: int, workspace=None, identity: bool = False,
-                     split_keys: int = 0, max_ctx: int = 0) -> None:
-    """Single-token items through the bfloat16 decode kernel; arguments as for ``attention``.
+                     split_keys: int = 0, max_ctx: int = 0, softcap: float = 0.0) -> None:
+    """Single-token items through the bfloat16 decode kernel; arguments as for ``attention``
+    (``softcap`` as for ``attention_prefill``).
     With more than one split it needs a float32 ``workspace``. ``identity``: item i is request i
     with its token in row i (no other items). ``split_keys`` > 0: every split takes that many
     keys at a fixed place; no context may then be longer than ``max_ctx`` <= n_splits * split_keys."""
@@ -1158,7 +1160,7 @@ def attention_decode(q, q_stride: int, out, k_cache, v_cache, block_tables, ctx_
             q.data_ptr(), int(q_stride), _ptr(out), out.shape[1], _ptr(k_cache), _ptr(v_cache), _ptr(block_tables),
             block_tables.shape[1], _ptr(ctx_lens), _ptr(cu_q), _ptr(items), n_items, nh, nkv, block_size, n_splits,
             window, float(scale), _ptr(workspace), ws_floats, _zero_row(out.device), int(bool(identity)),
-            int(split_keys), int(max_ctx), _stream()),
+            int(split_keys), int(max_ctx), float(softcap), _stream()),
         "attention_decode_bf16",
     )
 

@@ -70,8 +70,10 @@ class GatedAttention(Part):
         """Do the kernels for plain grouped attention take these heads? bfloat16, keys and values
         of one size that they are built for."""
         s = self.spec
+        # (the product's rows are padded to 16 bytes when the part is bound; those kernels know a
+        # window and a cap on the scores, but no kept first positions)
         return (dtype == torch.bfloat16 and s.key_dim == s.value_dim and s.key_dim % 32 == 0 and 32 <= s.key_dim <= 256
-                and self.in_width % 8 == 0 and not s.keep_first and s.softcap is None)
+                and not s.keep_first)
 
     def kernel_libraries(self) -> list:
         # the library of plain grouped attention is loaded (and, if missing, built) when the part is
@@ -174,7 +176,7 @@ class GatedAttention(Part):
             q=q, q_stride=q.shape[1], out=out, k_cache=k_plane, v_cache=v_plane,
             block_tables=ctx.block_tables[cache.group], ctx_lens=ctx.ctx_lens, cu_q=ctx.cu_q,
             nh=nh, nkv=nkv, hd=hd, block_size=cache.block_size, window=s.window or 0,
-            scale=s.scale, n_tokens=T, n_requests=ctx.num_requests,
+            scale=s.scale, n_tokens=T, n_requests=ctx.num_requests, softcap=s.softcap or 0.0,
         )
         if plan.n_wide:
             workspace = None

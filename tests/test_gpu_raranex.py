@@ -109,6 +109,38 @@ def test_capped_attention_whole_in_portions_and_token_by_token(dtype, shape):
         close(_step_through(part, part.cache_need(), x, cuts, dtype), want, dtype)
 
 
+@pytest.mark.parametrize("kind", ["window", "capped"])
+@pytest.mark.parametrize("shape", [(8, 2, 64, 64), (4, 1, 128, 128), (6, 3, 64, 128), (16, 2, 128, 64)])
+def test_the_attention_kernels_agree_on_long_requests(kind, shape):
+    """bfloat16, 700 tokens: the matrix-core kernels (for paged rows; for plain grouped heads where
+    keys and values have one size and nothing is kept) against the plain-arithmetic kernel on the
+    same steps and against the plain implementation, with the keys of single tokens and short
+    portions cut into runs (a card of 256 compute units is what the plan sizes them by)."""
+    heads, kv_heads, dim, vdim = shape
+    hidden, T, dtype = 64, 700, torch.bfloat16
+    if kind == "window":
+        spec = _window_spec(hidden, heads, kv_heads, dim, vdim, 130, 70, 32)
+        sizes, oracle = _window_sizes(spec), plain.window_attention
+    else:
+        spec = _capped_spec(hidden, heads, kv_heads, dim, vdim, softcap=3.0, coef=0.3, every=64)
+        sizes, oracle = _capped_sizes(spec), plain.capped_attention
+    x = torch.randn(T, hidden, generator=torch.Generator().manual_seed(16)).to(dtype)
+    outs = {}
+    for kernel in ("fast", "arithmetic"):
+        part = build_part(spec)
+        w = bind(part, dtype, seed=3, matrix_std=0.2)
+        assert part.plain == (kind == "capped" and dim == vdim) and part.rows_mfma == (not part.plain)
+        if kernel == "arithmetic":
+            part.plain = part.rows_mfma = False
+            part.run = ops.rows_attention_tokens_per_item(heads, kv_heads, 1)
+        for cuts in ([T], [600, 5, 2, 1, 1, 60] + [1] * 31):
+            got = _step_through(part, part.cache_need(), x, cuts, dtype, block_size=16, num_blocks=64, compute_units=256)
+            outs[(kernel, len(cuts))] = got
+    want = oracle(x.double(), _attention_names(w, spec), "", sizes, EPS)
+    for got in outs.values():
+        close(got, want, dtype)
+
+
 def test_the_attention_options_each_matter():
     """Every option of the two mixers switched off or changed by itself moves the output: the cap,
     the query's factor and its period, the kept tokens, the window, the order of norm and rotation
