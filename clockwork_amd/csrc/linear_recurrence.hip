@@ -261,6 +261,7 @@ struct SegParams {
   float* added;           // [n_segments, heads, dim, vdim]
   float* seg_decay;       // [n_segments, heads, dim]
   float* raw;             // [T, heads * vdim] outputs before norm and gate
+  float* own;             // [T, heads]: with a bonus, sum over d of q_d bonus_d k_d
   void* out;
   int heads, dim, vdim, rank, n_slots, n_tokens;
   float q_scale, inv_tau, eps;
@@ -319,6 +320,13 @@ __global__ __launch_bounds__(256) void lrs_prepare_kernel(SegParams p) {
     p.dec[idx] = lr_decay(z, p.form.decay_kind, p.inv_tau);
     p.qf[idx] = cw_to_float(row[p.q_off + c]) * p.q_scale;
     p.kf[idx] = cw_to_float(row[p.k_off + c]);
+    if (p.form.bonus && c % p.dim == 0) {
+      // the first channel's thread of a (token, head) sums the token's own share over the head's channels
+      float own = 0.0f;
+      for (int d = 0; d < p.dim; ++d)
+        own += cw_to_float(row[p.q_off + c + d]) * p.q_scale * p.form.bonus[c + d] * cw_to_float(row[p.k_off + c + d]);
+      p.own[t * p.heads + c / p.dim] = own;
+    }
   }
 }
 
@@ -367,6 +375,9 @@ __global__ __launch_bounds__(256) void lrs_walk_kernel(SegParams p) {
     if (MODE == 1) Qt[i] = p.qf[at];
   }
   __syncthreads();
+  // with a bonus the token's own share of its output is one number a token whatever the state's
+  // column, (sum over d of q_d bonus_d k_d) v: the prepare kernel has left the sums in ``own``
+  const bool reads_before = MODE == 1 && p.form.bonus != nullptr;   // the output reads the state before the token joins it
   for (int t = 0; t < nt; ++t) {
     const int64_t row = row0 + t;
     const float* a = As + t * D;
@@ -374,33 +385,37 @@ __global__ __launch_bounds__(256) void lrs_walk_kernel(SegParams p) {
     const float* q = Qt + t * D;
     const float vv = cw_to_float(proj[row * p.stride + p.v_off + h * V + vc]);
     float o0 = 0.0f, o1 = 0.0f, o2 = 0.0f, o3 = 0.0f;
-    if (MODE == 1 && p.form.bonus) {
-      // the output reads the state before the token joins it, and the token through the bonus
-      const float* bn = p.form.bonus + h * D;
+    if (reads_before) {
+      o0 = p.own[row * p.heads + h] * vv;
 #pragma unroll
       for (int d = 0; d < DIM; d += 4) {
         if (d < D) {
-          o0 += q[d] * (S[d] + bn[d] * k[d] * vv);
-          o1 += q[d + 1] * (S[d + 1] + bn[d + 1] * k[d + 1] * vv);
-          o2 += q[d + 2] * (S[d + 2] + bn[d + 2] * k[d + 2] * vv);
-          o3 += q[d + 3] * (S[d + 3] + bn[d + 3] * k[d + 3] * vv);
-        }
-      }
-    }
-#pragma unroll
-    for (int d = 0; d < DIM; d += 4) {
-      if (d < D) {  // D is a multiple of 4 here (the host sees to it)
-        S[d] = a[d] * S[d] + k[d] * vv;
-        S[d + 1] = a[d + 1] * S[d + 1] + k[d + 1] * vv;
-        S[d + 2] = a[d + 2] * S[d + 2] + k[d + 2] * vv;
-        S[d + 3] = a[d + 3] * S[d + 3] + k[d + 3] * vv;
-        if (MODE == 1 && !p.form.bonus) {
           o0 += q[d] * S[d];
           o1 += q[d + 1] * S[d + 1];
           o2 += q[d + 2] * S[d + 2];
           o3 += q[d + 3] * S[d + 3];
-        } else if (MODE == 0 && threadIdx.x == 0 && blockIdx.z == 0) {
-          A[d] *= a[d]; A[d + 1] *= a[d + 1]; A[d + 2] *= a[d + 2]; A[d + 3] *= a[d + 3];
+          S[d] = a[d] * S[d] + k[d] * vv;
+          S[d + 1] = a[d + 1] * S[d + 1] + k[d + 1] * vv;
+          S[d + 2] = a[d + 2] * S[d + 2] + k[d + 2] * vv;
+          S[d + 3] = a[d + 3] * S[d + 3] + k[d + 3] * vv;
+        }
+      }
+    } else {
+#pragma unroll
+      for (int d = 0; d < DIM; d += 4) {
+        if (d < D) {  // D is a multiple of 4 here (the host sees to it)
+          S[d] = a[d] * S[d] + k[d] * vv;
+          S[d + 1] = a[d + 1] * S[d + 1] + k[d + 1] * vv;
+          S[d + 2] = a[d + 2] * S[d + 2] + k[d + 2] * vv;
+          S[d + 3] = a[d + 3] * S[d + 3] + k[d + 3] * vv;
+          if (MODE == 1) {
+            o0 += q[d] * S[d];
+            o1 += q[d + 1] * S[d + 1];
+            o2 += q[d + 2] * S[d + 2];
+            o3 += q[d + 3] * S[d + 3];
+          } else if (threadIdx.x == 0 && blockIdx.z == 0) {
+            A[d] *= a[d]; A[d + 1] *= a[d + 1]; A[d + 2] *= a[d + 2]; A[d + 3] *= a[d + 3];
+          }
         }
       }
     }
@@ -474,9 +489,10 @@ CW_EXPORT int cw_linear_recurrence_segments_supported(int dim, int vdim) {
 }
 
 // floats of workspace: dec, qf, kf [T, heads * dim] each, added [segments, heads, dim, vdim],
-// seg_decay [segments, heads, dim], raw [T, heads * vdim]
+// seg_decay [segments, heads, dim], raw [T, heads * vdim], own [T, heads]
 CW_EXPORT int64_t cw_linear_recurrence_segments_workspace_floats(int n_tokens, int n_segments, int heads, int dim, int vdim) {
-  return 3 * (int64_t)n_tokens * heads * dim + (int64_t)n_segments * heads * dim * (vdim + 1) + (int64_t)n_tokens * heads * vdim;
+  return 3 * (int64_t)n_tokens * heads * dim + (int64_t)n_segments * heads * dim * (vdim + 1) + (int64_t)n_tokens * heads * vdim +
+         (int64_t)n_tokens * heads;
 }
 
 CW_EXPORT int cw_linear_recurrence_segments(int dtype, const void* proj, int64_t stride, int q_off, int k_off, int v_off,
@@ -513,6 +529,7 @@ CW_EXPORT int cw_linear_recurrence_segments(int dtype, const void* proj, int64_t
   p.added = p.kf + THD;
   p.seg_decay = p.added + (int64_t)n_segments * heads * dim * vdim;
   p.raw = p.seg_decay + (int64_t)n_segments * heads * dim;
+  p.own = p.raw + (int64_t)n_tokens * heads * vdim;
   int64_t pb = (THD + 255) / 256;
   if (pb > 65536) pb = 65536;
   p.seg_tokens = seg_tokens;
