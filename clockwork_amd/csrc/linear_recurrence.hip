@@ -261,7 +261,6 @@ struct SegParams {
   float* added;           // [n_segments, heads, dim, vdim]
   float* seg_decay;       // [n_segments, heads, dim]
   float* raw;             // [T, heads * vdim] outputs before norm and gate
-  float* own;             // [T, heads]: with a bonus, sum over d of q_d bonus_d k_d
   void* out;
   int heads, dim, vdim, rank, n_slots, n_tokens;
   float q_scale, inv_tau, eps;
@@ -320,13 +319,6 @@ __global__ __launch_bounds__(256) void lrs_prepare_kernel(SegParams p) {
     p.dec[idx] = lr_decay(z, p.form.decay_kind, p.inv_tau);
     p.qf[idx] = cw_to_float(row[p.q_off + c]) * p.q_scale;
     p.kf[idx] = cw_to_float(row[p.k_off + c]);
-    if (p.form.bonus && c % p.dim == 0) {
-      // the first channel's thread of a (token, head) sums the token's own share over the head's channels
-      float own = 0.0f;
-      for (int d = 0; d < p.dim; ++d)
-        own += cw_to_float(row[p.q_off + c + d]) * p.q_scale * p.form.bonus[c + d] * cw_to_float(row[p.k_off + c + d]);
-      p.own[t * p.heads + c / p.dim] = own;
-    }
   }
 }
 
@@ -376,7 +368,19 @@ __global__ __launch_bounds__(256) void lrs_walk_kernel(SegParams p) {
   }
   __syncthreads();
   // with a bonus the token's own share of its output is one number a token whatever the state's
-  // column, (sum over d of q_d bonus_d k_d) v: the prepare kernel has left the sums in ``own``
+  // column, (sum over d of q_d bonus_d k_d) v: lane t of every wave sums token t's, once a segment,
+  // and hands it to the others when the token's turn comes (a segment has at most 64 tokens)
+  float own = 0.0f;
+  if (MODE == 1 && p.form.bonus) {
+    const int lane = threadIdx.x & 63;
+    if (lane < nt) {
+      const float* bn = p.form.bonus + h * D;
+      for (int i = 0; i < D; ++i) {
+        const int d = (i + lane) % D;   // every lane a bank of its own
+        own += Qt[lane * D + d] * bn[d] * Kt[lane * D + d];
+      }
+    }
+  }
   const bool reads_before = MODE == 1 && p.form.bonus != nullptr;   // the output reads the state before the token joins it
   for (int t = 0; t < nt; ++t) {
     const int64_t row = row0 + t;
@@ -386,7 +390,7 @@ __global__ __launch_bounds__(256) void lrs_walk_kernel(SegParams p) {
     const float vv = cw_to_float(proj[row * p.stride + p.v_off + h * V + vc]);
     float o0 = 0.0f, o1 = 0.0f, o2 = 0.0f, o3 = 0.0f;
     if (reads_before) {
-      o0 = p.own[row * p.heads + h] * vv;
+      o0 = __shfl(own, t, 64) * vv;
 #pragma unroll
       for (int d = 0; d < DIM; d += 4) {
         if (d < D) {
@@ -489,10 +493,9 @@ CW_EXPORT int cw_linear_recurrence_segments_supported(int dim, int vdim) {
 }
 
 // floats of workspace: dec, qf, kf [T, heads * dim] each, added [segments, heads, dim, vdim],
-// seg_decay [segments, heads, dim], raw [T, heads * vdim], own [T, heads]
+// seg_decay [segments, heads, dim], raw [T, heads * vdim]
 CW_EXPORT int64_t cw_linear_recurrence_segments_workspace_floats(int n_tokens, int n_segments, int heads, int dim, int vdim) {
-  return 3 * (int64_t)n_tokens * heads * dim + (int64_t)n_segments * heads * dim * (vdim + 1) + (int64_t)n_tokens * heads * vdim +
-         (int64_t)n_tokens * heads;
+  return 3 * (int64_t)n_tokens * heads * dim + (int64_t)n_segments * heads * dim * (vdim + 1) + (int64_t)n_tokens * heads * vdim;
 }
 
 CW_EXPORT int cw_linear_recurrence_segments(int dtype, const void* proj, int64_t stride, int q_off, int k_off, int v_off,
@@ -515,7 +518,7 @@ CW_EXPORT int cw_linear_recurrence_segments(int dtype, const void* proj, int64_t
     return CW_ERR_ARG;
   if (!cw_linear_recurrence_segments_supported(dim, vdim)) return CW_ERR_SIZE;
   if (heads > 65535 || (vdim + 63) / 64 > 65535) return CW_ERR_SIZE;
-  if (seg_tokens < 1 || (int64_t)3 * seg_tokens * dim * 4 > 48 * 1024) return CW_ERR_SIZE;
+  if (seg_tokens < 1 || (int64_t)3 * seg_tokens * dim * 4 > 48 * 1024 || (bonus && seg_tokens > 64)) return CW_ERR_SIZE;
   if (n_requests == 0 || n_tokens == 0 || n_segments == 0) return CW_OK;
   SegParams p;
   p.proj = proj; p.stride = stride; p.q_off = q_off; p.k_off = k_off; p.v_off = v_off; p.g_off = g_off; p.u_off = u_off;
@@ -529,7 +532,6 @@ CW_EXPORT int cw_linear_recurrence_segments(int dtype, const void* proj, int64_t
   p.added = p.kf + THD;
   p.seg_decay = p.added + (int64_t)n_segments * heads * dim * vdim;
   p.raw = p.seg_decay + (int64_t)n_segments * heads * dim;
-  p.own = p.raw + (int64_t)n_tokens * heads * vdim;
   int64_t pb = (THD + 255) / 256;
   if (pb > 65536) pb = 65536;
   p.seg_tokens = seg_tokens;
