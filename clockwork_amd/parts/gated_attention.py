@@ -127,7 +127,7 @@ class GatedAttention(Part):
         plan = ctx.plans.get(key)
         if plan is None:
             items, n_items = query_runs(ctx, self.run)
-            # every item's keys are cut into runs where the step would leave most of the card idle
+            # every item's keys are cut into runs where the step would leave most of the compute units idle
             longest = longest_key_range(ctx, s.window) + (s.keep_first if s.window is not None else 0)
             runs = ops.rows_mfma_key_runs(n_items, longest, s.num_heads, s.num_kv_heads, s.key_dim, s.value_dim, 1,
                                           ctx.num_compute_units)

@@ -115,7 +115,7 @@ def test_the_attention_kernels_agree_on_long_requests(kind, shape):
     """bfloat16, 700 tokens: the matrix-core kernels (for paged rows; for plain grouped heads where
     keys and values have one size and nothing is kept) against the plain-arithmetic kernel on the
     same steps and against the plain implementation, with the keys of single tokens and short
-    portions cut into runs (a card of 256 compute units is what the plan sizes them by)."""
+    portions cut into runs (a GPU of 256 compute units is what the plan sizes them by)."""
     heads, kv_heads, dim, vdim = shape
     hidden, T, dtype = 64, 700, torch.bfloat16
     if kind == "window":
