@@ -73,7 +73,9 @@ CUTS = lambda T: ([T], [5, 1, 1, 17, 2, 1, 2, T - 29], [1] * T)  # noqa: E731
 # and one of 1, more kept tokens than the window holds, rotation of all, a part and nothing
 WINDOW_SHAPES = [(6, 2, 16, 24, 9, 3, 8, 96), (3, 1, 40, 8, 17, 1, 40, 100), (5, 5, 12, 20, 1, 4, 12, 64), (1, 1, 2, 1, 16, 0, 2, 48),
                  (4, 2, 24, 24, 300, 7, 0, 64), (20, 2, 8, 16, 12, 20, 4, 64), (8, 2, 64, 64, 33, 5, 32, 128),
-                 (4, 4, 128, 64, 25, 2, 128, 64), (6, 3, 64, 64, 5, 9, 64, 66), (2, 1, 96, 48, 40, 40, 64, 72)]
+                 (4, 4, 128, 64, 25, 2, 128, 64), (6, 3, 64, 64, 5, 9, 64, 66), (2, 1, 96, 48, 40, 40, 64, 72),
+                 # nothing kept and keys and values of one size: in bfloat16 the kernels of plain grouped attention
+                 (8, 2, 64, 64, 33, 0, 32, 128), (4, 4, 32, 32, 9, 0, 32, 64), (6, 1, 96, 96, 20, 0, 48, 72), (2, 2, 256, 256, 7, 0, 64, 64)]
 
 
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
@@ -92,7 +94,7 @@ def test_window_attention_whole_in_portions_and_token_by_token(dtype, shape):
 
 # heads, kv_heads, dim, vdim, hidden
 CAPPED_SHAPES = [(8, 1, 24, 12, 96), (3, 3, 40, 8, 100), (1, 1, 2, 1, 48), (20, 2, 8, 16, 64), (8, 2, 64, 64, 128), (4, 4, 128, 64, 64),
-                 (2, 1, 96, 48, 72), (5, 5, 12, 130, 64)]
+                 (2, 1, 96, 48, 72), (5, 5, 12, 130, 64), (6, 2, 32, 32, 64), (3, 1, 160, 160, 40), (4, 2, 64, 256, 64), (16, 1, 16, 16, 64)]
 
 
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
